@@ -1,0 +1,387 @@
+// C ABI of the CATS sparse-MLP decode kernels (declared in include/cats_gemv.h): argument checks,
+// workspace carving, launch-shape selection and dispatch on dtype.  No allocation, no synchronisation
+// (cats_read_count excepted), everything on the caller's stream.
+#include <hip/hip_runtime.h>
+#include <string.h>
+
+#include "cats_gemv.h"
+#include "cats_launch.h"
+
+namespace cats {
+
+// Per-dtype launchers live in cats_inst.hip.
+template <> hipError_t launch_rows<F16>(int, int, const RowsArgs&, hipStream_t);
+template <> hipError_t launch_rows<BF16>(int, int, const RowsArgs&, hipStream_t);
+template <> hipError_t launch_rows<F32>(int, int, const RowsArgs&, hipStream_t);
+template <> hipError_t launch_down<F16>(int, bool, const DownArgs&, int, hipStream_t);
+template <> hipError_t launch_down<BF16>(int, bool, const DownArgs&, int, hipStream_t);
+template <> hipError_t launch_down<F32>(int, bool, const DownArgs&, int, hipStream_t);
+
+namespace {
+
+Tuning g_tuning = {0, 0, 0};
+
+constexpr int kMaxSlabs = 128;
+constexpr size_t kCounterBytes = 1024;  // done[128] | arrive | pad
+
+__global__ void fill_zero_kernel(u32x4* p, size_t n16) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) p[i] = zero4();
+}
+
+// (nb, I) flag bytes -> ceil(I/8) mask bytes, bit j = OR over the batch of flag[b, j].
+__global__ void pack_flags_kernel(const uint8_t* flag, int nb, int I, uint8_t* mask, int nbytes) {
+  const int byte = blockIdx.x * blockDim.x + threadIdx.x;
+  if (byte >= nbytes) return;
+  uint32_t bits = 0;
+  for (int e = 0; e < 8; e++) {
+    const int j = byte * 8 + e;
+    if (j < I) {
+      uint32_t on = 0;
+      for (int b = 0; b < nb; b++) on |= flag[(size_t)b * I + j] != 0 ? 1u : 0u;
+      bits |= on << e;
+    }
+  }
+  mask[byte] = (uint8_t)bits;
+}
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct WsLayout {
+  size_t counters, mask, z32, zt, y32, atmp, total;
+};
+
+// The carving depends on (H, I) only -- every region is sized for CATS_MAX_BATCH rows -- so calls with
+// different batch sizes can share one workspace and the regions that must stay zero (counters, y32) never
+// move onto bytes another call has dirtied.
+WsLayout ws_layout(int H, int I) {
+  WsLayout l;
+  const int B = CATS_MAX_BATCH;
+  size_t o = 0;
+  l.counters = o; o += kCounterBytes;
+  l.y32 = o;      o += align_up((size_t)B * H * 4, 256);
+  l.mask = o;     o += align_up((size_t)((I + 63) / 64) * 8, 256);
+  l.z32 = o;      o += align_up((size_t)B * I * 4, 256);
+  l.zt = o;       o += align_up((size_t)B * I * 4, 256);
+  l.atmp = o;     o += align_up((size_t)B * I * 4, 256);
+  l.total = o;
+  return l;
+}
+
+inline int elem_size(int dtype) { return dtype == CATS_F32 ? 4 : 2; }
+inline int vec_elems(int dtype) { return dtype == CATS_F32 ? 4 : 8; }
+inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// float -> fp16 bits, round to nearest even (host side, for the threshold).
+uint16_t f32_to_f16_bits(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  x &= 0x7fffffffu;
+  if (x > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);           // NaN
+  if (x >= 0x47800000u) return (uint16_t)(sign | 0x7c00u);          // >= 65536 -> inf (65520 rounds up below)
+  if (x < 0x38800000u) {                                             // below the smallest normal half
+    if (x < 0x33000000u) return (uint16_t)sign;                      // < 2^-25 -> 0
+    const int e = (int)(x >> 23);                                     // biased fp32 exponent
+    uint32_t m = (x & 0x7fffffu) | 0x800000u;                         // 24-bit significand
+    const int shift = 126 - e;                                        // 14..24: bits dropped to reach 2^-24 units
+    const uint32_t half = 1u << (shift - 1);
+    const uint32_t rem = m & ((1u << shift) - 1u);
+    m >>= shift;
+    if (rem > half || (rem == half && (m & 1u))) m++;
+    return (uint16_t)(sign | m);
+  }
+  uint32_t h = ((x - 0x38000000u) >> 13);                            // rebias exponent, keep 10 mantissa bits
+  const uint32_t rem = x & 0x1fffu;
+  if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h++;            // may carry into the exponent (and to inf)
+  return (uint16_t)(sign | h);
+}
+
+float f16_bits_to_f32(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu, x;
+  if (e == 0) {
+    if (m == 0) {
+      x = sign;
+    } else {
+      int s = 0;
+      while (!(m & 0x400u)) { m <<= 1; s++; }
+      x = sign | ((uint32_t)(113 - s) << 23) | ((m & 0x3ffu) << 13);
+    }
+  } else if (e == 31) {
+    x = sign | 0x7f800000u | (m << 13);
+  } else {
+    x = sign | ((e + 112) << 23) | (m << 13);
+  }
+  float f;
+  memcpy(&f, &x, 4);
+  return f;
+}
+
+float round_through(int dtype, float t) {
+  if (dtype == CATS_F16) return f16_bits_to_f32(f32_to_f16_bits(t));
+  if (dtype == CATS_BF16) {
+    uint32_t u;
+    memcpy(&u, &t, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return t;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    u &= 0xffff0000u;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+  }
+  return t;
+}
+
+int batch_template(int B) { return B <= 1 ? 1 : (B <= 2 ? 2 : (B <= 4 ? 4 : 8)); }
+
+int check_common(int B, int H, int I, int dtype) {
+  if (dtype != CATS_F16 && dtype != CATS_BF16 && dtype != CATS_F32) return CATS_ERR_DTYPE;
+  if (B < 1 || B > CATS_MAX_BATCH) return CATS_ERR_BATCH;
+  if (H <= 0 || I <= 0) return CATS_ERR_SHAPE;
+  if (((size_t)H * elem_size(dtype)) % 16 != 0) return CATS_ERR_ALIGN;
+  return CATS_OK;
+}
+
+void fill_rows(RowsArgs& a, const void* x, const void* w, int K, int N, int nb, int dtype) {
+  memset(&a, 0, sizeof(a));
+  a.x = (const u32x4*)x;
+  a.w = (const u32x4*)w;
+  a.K = K;
+  a.N = N;
+  a.nb = nb;
+  const int vec = vec_elems(dtype);
+  a.row_vecs = K / vec;
+  a.nch = (a.row_vecs + kWave - 1) / kWave;
+}
+
+int do_rows(int mode, int dtype, const RowsArgs& a, hipStream_t s) {
+  const int bt = batch_template(a.nb);
+  hipError_t e;
+  if (dtype == CATS_F16) e = launch_rows<F16>(mode, bt, a, s);
+  else if (dtype == CATS_BF16) e = launch_rows<BF16>(mode, bt, a, s);
+  else e = launch_rows<F32>(mode, bt, a, s);
+  return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+}
+
+// Sparse down over mask words already in the workspace.
+int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_out, int32_t* count_out, int B, int H, int I,
+            int dtype, char* ws, const WsLayout& l, hipStream_t s) {
+  DownArgs d;
+  memset(&d, 0, sizeof(d));
+  d.wd = (const u32x4*)wdown_t;
+  d.z = z;
+  d.mask = (const uint64_t*)(ws + l.mask);
+  d.y32 = y32;
+  d.y_out = y_out;
+  d.done = (uint32_t*)(ws + l.counters);
+  d.count_out = count_out;
+  d.H = H; d.I = I; d.nb = B;
+  d.row_vecs = H / vec_elems(dtype);
+  d.nslab = (d.row_vecs + kWave - 1) / kWave;
+  d.nwords = (I + 63) / 64;
+  if (d.nslab > kMaxSlabs || I > CATS_MAX_INTERMEDIATE) return CATS_ERR_SHAPE;
+  int ngroup = g_tuning.down_groups > 0 ? g_tuning.down_groups : 256 / d.nslab;
+  if (ngroup < 1) ngroup = 1;
+  if (ngroup > I) ngroup = I;
+  d.ngroup = ngroup;
+  d.ncap = (I + ngroup - 1) / ngroup + 1;
+  int block = g_tuning.down_block > 0 ? g_tuning.down_block : 1024;
+  if (block < 64) block = 64;
+  if (block > 1024) block = 1024;
+  block = block / 64 * 64;
+  const int bt = batch_template(B);
+  hipError_t e;
+  if (dtype == CATS_F16) e = launch_down<F16>(bt, zf32, d, block, s);
+  else if (dtype == CATS_BF16) e = launch_down<BF16>(bt, zf32, d, block, s);
+  else e = launch_down<F32>(bt, zf32, d, block, s);
+  return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+}
+
+int check_ws(const void* ws, size_t ws_bytes, int H, int I, WsLayout& l) {
+  l = ws_layout(H, I);
+  if (ws == nullptr || ws_bytes < l.total || ((uintptr_t)ws & 255u) != 0) return CATS_ERR_WORKSPACE;
+  return CATS_OK;
+}
+
+}  // namespace
+}  // namespace cats
+
+using namespace cats;
+
+extern "C" {
+
+int cats_version(void) { return 100; }
+
+const char* cats_status_string(int status) {
+  switch (status) {
+    case CATS_OK: return "ok";
+    case CATS_ERR_DTYPE: return "unsupported dtype (expected 0=fp16, 1=bf16, 2=fp32)";
+    case CATS_ERR_SHAPE: return "unsupported shape (H, I must be positive; I <= 65536; H <= 128 slabs of 64 x 16 bytes)";
+    case CATS_ERR_ALIGN: return "pointer or row pitch not 16-byte aligned";
+    case CATS_ERR_BATCH: return "unsupported batch (1..8 rows)";
+    case CATS_ERR_NULL: return "required pointer is NULL";
+    case CATS_ERR_WORKSPACE: return "workspace missing, misaligned (256 bytes) or smaller than cats_workspace_bytes()";
+    case CATS_ERR_LAUNCH: return "HIP kernel launch failed";
+  }
+  return "unknown status";
+}
+
+int cats_set_tuning(int gate_variant, int down_groups, int down_block) {
+  g_tuning.gate_variant = gate_variant;
+  g_tuning.down_groups = down_groups;
+  g_tuning.down_block = down_block;
+  return CATS_OK;
+}
+
+size_t cats_workspace_bytes(int B, int H, int I) {
+  if (B < 1 || H < 1 || I < 1) return 0;
+  return ws_layout(H, I).total;
+}
+
+int cats_workspace_init(void* ws, size_t ws_bytes, void* stream) {
+  if (ws == nullptr) return CATS_ERR_NULL;
+  if (((uintptr_t)ws & 255u) != 0 || ws_bytes % 16 != 0) return CATS_ERR_WORKSPACE;
+  const size_t n16 = ws_bytes / 16;
+  int grid = (int)((n16 + 255) / 256);
+  if (grid > 2048) grid = 2048;
+  if (grid < 1) grid = 1;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (u32x4*)ws, n16);
+  return hipGetLastError() == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+}
+
+int cats_gate_flag(const void* x, const void* wgate, void* a_out, uint8_t* flag_out, int B, int H, int I, int dtype,
+                   float threshold, void* stream) {
+  int st = check_common(B, H, I, dtype);
+  if (st) return st;
+  if (!x || !wgate || (!a_out && !flag_out)) return CATS_ERR_NULL;
+  if (!aligned16(x) || !aligned16(wgate)) return CATS_ERR_ALIGN;
+  RowsArgs a;
+  fill_rows(a, x, wgate, H, I, B, dtype);
+  a.a_out = a_out;
+  a.flag_out = flag_out;
+  a.t = round_through(dtype, threshold);
+  return do_rows(kGate, dtype, a, (hipStream_t)stream);
+}
+
+int cats_gate_compact(const void* x, const void* wgate, void* vals_out, int64_t* idx_out, int32_t* count_out, int H, int I,
+                      int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
+  int st = check_common(1, H, I, dtype);
+  if (st) return st;
+  if (!x || !wgate || !idx_out || !count_out) return CATS_ERR_NULL;
+  if (!aligned16(x) || !aligned16(wgate)) return CATS_ERR_ALIGN;
+  WsLayout l;
+  st = check_ws(ws, ws_bytes, H, I, l);
+  if (st) return st;
+  RowsArgs a;
+  fill_rows(a, x, wgate, H, I, 1, dtype);
+  a.a_out = (char*)ws + l.atmp;
+  a.mask_out = (uint8_t*)ws + l.mask;
+  a.arrive = (uint32_t*)((char*)ws + l.counters + 512);
+  a.idx_out = idx_out;
+  a.vals_out = vals_out;
+  a.count_out = count_out;
+  a.t = round_through(dtype, threshold);
+  return do_rows(kGate, dtype, a, (hipStream_t)stream);
+}
+
+int cats_read_count(const int32_t* count_dev, void* stream) {
+  if (!count_dev) return -1;
+  if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return -1;
+  int32_t v = -1;
+  if (hipMemcpy(&v, count_dev, sizeof(v), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+  return v;
+}
+
+int cats_up_flag(const void* x, const void* wup, const void* a_in, const uint8_t* flag, void* out, int out_is_f32, int B,
+                 int H, int I, int dtype, void* stream) {
+  int st = check_common(B, H, I, dtype);
+  if (st) return st;
+  if (!x || !wup || !a_in || !flag || !out) return CATS_ERR_NULL;
+  if (!aligned16(x) || !aligned16(wup)) return CATS_ERR_ALIGN;
+  RowsArgs a;
+  fill_rows(a, x, wup, H, I, B, dtype);
+  a.a_in = a_in;
+  a.flag_in = flag;
+  if (out_is_f32) a.z32_out = (float*)out; else a.zt_out = out;
+  return do_rows(kUp, dtype, a, (hipStream_t)stream);
+}
+
+int cats_down_flag(const void* z, const void* wdown_t, const uint8_t* flag, float* y_f32, void* y_out, int B, int H, int I,
+                   int dtype, void* ws, size_t ws_bytes, void* stream) {
+  int st = check_common(B, H, I, dtype);
+  if (st) return st;
+  if (!z || !wdown_t || !flag || ((y_f32 == nullptr) == (y_out == nullptr))) return CATS_ERR_NULL;
+  if (!aligned16(wdown_t)) return CATS_ERR_ALIGN;
+  WsLayout l;
+  st = check_ws(ws, ws_bytes, H, I, l);
+  if (st) return st;
+  const int nbytes = (I + 7) / 8;
+  hipLaunchKernelGGL(pack_flags_kernel, dim3((nbytes + 255) / 256), dim3(256), 0, (hipStream_t)stream, flag, B, I,
+                     (uint8_t*)ws + l.mask, nbytes);
+  if (hipGetLastError() != hipSuccess) return CATS_ERR_LAUNCH;
+  float* acc = y_f32 ? y_f32 : (float*)((char*)ws + l.y32);
+  return do_down(z, false, wdown_t, acc, y_out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
+}
+
+int cats_gate_up(const void* x, const void* wgate, const void* wup, void* out, uint8_t* flag_out, int B, int H, int I,
+                 int dtype, float threshold, void* stream) {
+  int st = check_common(B, H, I, dtype);
+  if (st) return st;
+  if (!x || !wgate || !wup || !out) return CATS_ERR_NULL;
+  if (!aligned16(x) || !aligned16(wgate) || !aligned16(wup)) return CATS_ERR_ALIGN;
+  RowsArgs a;
+  fill_rows(a, x, wgate, H, I, B, dtype);
+  a.w2 = (const u32x4*)wup;
+  a.zt_out = out;
+  a.flag_out = flag_out;
+  a.t = round_through(dtype, threshold);
+  return do_rows(kGateUp, dtype, a, (hipStream_t)stream);
+}
+
+int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, float* y_f32,
+             uint8_t* flag_out, int32_t* count_out, int B, int H, int I, int dtype, float threshold, void* ws,
+             size_t ws_bytes, void* stream) {
+  int st = check_common(B, H, I, dtype);
+  if (st) return st;
+  if (!x || !wgate || !wup || !wdown_t || ((y_f32 == nullptr) == (y_out == nullptr))) return CATS_ERR_NULL;
+  if (!aligned16(x) || !aligned16(wgate) || !aligned16(wup) || !aligned16(wdown_t)) return CATS_ERR_ALIGN;
+  WsLayout l;
+  st = check_ws(ws, ws_bytes, H, I, l);
+  if (st) return st;
+  RowsArgs a;
+  fill_rows(a, x, wgate, H, I, B, dtype);
+  a.w2 = (const u32x4*)wup;
+  a.z32_out = (float*)((char*)ws + l.z32);
+  a.mask_out = (uint8_t*)ws + l.mask;
+  a.flag_out = flag_out;
+  a.t = round_through(dtype, threshold);
+  st = do_rows(kGateUp, dtype, a, (hipStream_t)stream);
+  if (st) return st;
+  float* acc = y_f32 ? y_f32 : (float*)((char*)ws + l.y32);
+  return do_down(a.z32_out, true, wdown_t, acc, y_out, count_out, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
+}
+
+int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out, int B, int H,
+                           int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
+  int st = check_common(B, H, I, dtype);
+  if (st) return st;
+  if (!x || !wgate || !wup || !wdown || !y_out) return CATS_ERR_NULL;
+  if (!aligned16(x) || !aligned16(wgate) || !aligned16(wup) || !aligned16(wdown)) return CATS_ERR_ALIGN;
+  if (((size_t)I * elem_size(dtype)) % 16 != 0) return CATS_ERR_ALIGN;
+  WsLayout l;
+  st = check_ws(ws, ws_bytes, H, I, l);
+  if (st) return st;
+  RowsArgs a;
+  fill_rows(a, x, wgate, H, I, B, dtype);
+  a.w2 = (const u32x4*)wup;
+  a.zt_out = (char*)ws + l.zt;
+  a.t = round_through(dtype, threshold);
+  st = do_rows(kGateUp, dtype, a, (hipStream_t)stream);
+  if (st) return st;
+  RowsArgs g;
+  fill_rows(g, (char*)ws + l.zt, wdown, I, H, B, dtype);
+  g.zt_out = y_out;
+  return do_rows(kGemv, dtype, g, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,101 @@
+// Kernel instantiations for one dtype.  Compiled three times (-DCATS_DT=F16 / BF16 / F32) so the
+// translation units build in parallel.
+#include "cats_launch.h"
+
+#ifndef CATS_DT
+#error "compile with -DCATS_DT=F16|BF16|F32"
+#endif
+
+namespace cats {
+
+namespace {
+
+constexpr int kR = 2;    // rows per wave per pass
+constexpr int kCB = 8;   // 64-lane chunks whose loads are issued together: 8 x 16 B per lane per row
+constexpr int kDownU = 8;  // rows in flight per lane in the down kernel
+
+// Workgroup width by batch: x is staged per workgroup, so wider batches share it across more waves.
+template <int B> struct WavesFor { static constexpr int value = B <= 2 ? 4 : (B == 4 ? 8 : 16); };
+
+template <class DT, int B, bool FULL, int MODE, bool XLDS>
+hipError_t launch_rows_one(const RowsArgs& a, hipStream_t stream) {
+  constexpr int WAVES = WavesFor<B>::value;
+  auto kern = rows_kernel<DT, B, kR, kCB, FULL, MODE, XLDS, WAVES>;
+  const int rows_per_block = WAVES * kR;
+  const int grid = (a.N + rows_per_block - 1) / rows_per_block;
+  const size_t lds = XLDS ? (size_t)B * ((a.nch + kCB - 1) / kCB * kCB) * kWave * sizeof(u32x4) : 0;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(WAVES * kWave), lds, stream, a);
+  return hipGetLastError();
+}
+
+template <class DT, int B>
+hipError_t launch_rows_b(int mode, const RowsArgs& a, hipStream_t stream) {
+  const size_t lds = (size_t)B * ((a.nch + kCB - 1) / kCB * kCB) * kWave * sizeof(u32x4);
+  const bool xlds = lds <= 128 * 1024;
+  const bool full = xlds && (a.K % (kWave * DT::VEC * kCB) == 0);
+  switch (mode) {
+    case kGate:
+      if (full) return launch_rows_one<DT, B, true, kGate, true>(a, stream);
+      if (xlds) return launch_rows_one<DT, B, false, kGate, true>(a, stream);
+      return launch_rows_one<DT, B, false, kGate, false>(a, stream);
+    case kGateUp:
+      if (full) return launch_rows_one<DT, B, true, kGateUp, true>(a, stream);
+      if (xlds) return launch_rows_one<DT, B, false, kGateUp, true>(a, stream);
+      return launch_rows_one<DT, B, false, kGateUp, false>(a, stream);
+    case kUp:
+      if (xlds) return launch_rows_one<DT, B, false, kUp, true>(a, stream);
+      return launch_rows_one<DT, B, false, kUp, false>(a, stream);
+    case kGemv:
+      if (xlds) return launch_rows_one<DT, B, false, kGemv, true>(a, stream);
+      return launch_rows_one<DT, B, false, kGemv, false>(a, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+template <class DT, int B, bool ZF32>
+hipError_t launch_down_one(const DownArgs& a, int block, hipStream_t stream) {
+  auto kern = down_kernel<DT, B, ZF32, kDownU>;
+  const int nwaves = block / kWave;
+  const size_t lds = ((size_t)a.ncap * (1 + B) + (size_t)nwaves * kWave * DT::VEC) * sizeof(float);
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, dim3(a.nslab * a.ngroup), dim3(block), lds, stream, a);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+template <>
+hipError_t launch_rows<CATS_DT>(int mode, int bt, const RowsArgs& a, hipStream_t stream) {
+  switch (bt) {
+    case 1: return launch_rows_b<CATS_DT, 1>(mode, a, stream);
+    case 2: return launch_rows_b<CATS_DT, 2>(mode, a, stream);
+    case 4: return launch_rows_b<CATS_DT, 4>(mode, a, stream);
+    case 8: return launch_rows_b<CATS_DT, 8>(mode, a, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+template <>
+hipError_t launch_down<CATS_DT>(int bt, bool zf32, const DownArgs& a, int block, hipStream_t stream) {
+#define CATS_DOWN_CASE(BB)                                                         \
+  case BB:                                                                         \
+    return zf32 ? launch_down_one<CATS_DT, BB, true>(a, block, stream)             \
+                : launch_down_one<CATS_DT, BB, false>(a, block, stream);
+  switch (bt) {
+    CATS_DOWN_CASE(1)
+    CATS_DOWN_CASE(2)
+    CATS_DOWN_CASE(4)
+    CATS_DOWN_CASE(8)
+  }
+#undef CATS_DOWN_CASE
+  return hipErrorInvalidValue;
+}
+
+}  // namespace cats

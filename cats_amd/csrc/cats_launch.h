@@ -1,0 +1,23 @@
+// Host-side launch interface between the C ABI (cats_api.hip) and the per-dtype kernel instantiations
+// (cats_inst.hip, compiled once per dtype).
+#pragma once
+#include <hip/hip_runtime.h>
+#include "cats_down.h"
+#include "cats_rows.h"
+
+namespace cats {
+
+struct Tuning {
+  int gate_variant;  // reserved for alternative gate kernels; 0 = default
+  int down_groups;   // 0 = default (about one workgroup per CU over all slabs)
+  int down_block;    // 0 = default (1024 threads)
+};
+
+// Returns hipSuccess or the launch error.  `mode` is a RowsMode; bt (1, 2, 4 or 8) the compile-time batch.
+template <class DT>
+hipError_t launch_rows(int mode, int bt, const RowsArgs& a, hipStream_t stream);
+
+template <class DT>
+hipError_t launch_down(int bt, bool zf32, const DownArgs& a, int block, hipStream_t stream);
+
+}  // namespace cats

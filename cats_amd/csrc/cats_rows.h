@@ -1,0 +1,272 @@
+// Row-streaming kernel: one wavefront owns R consecutive weight rows at a time, every lane issues
+// 128-bit streaming loads over the row, the dot products are accumulated in fp32 and folded across the
+// wave with DPP.  One template covers the four row-major passes of the CATS MLP:
+//
+//   kGate    a = SiLU(x . wgate[j]) ; flag = |a| > t ; optional mask words ; optional compact list
+//   kGateUp  the gate pass, then for rows that came out active the matching wup row:  z = a * (x . wup[j])
+//   kUp      flags and a are given; fetch wup rows with any flag set:                  out = a * (x . wup[j])
+//   kGemv    plain y = W x (the dense (H,I) down projection over the zero-filled intermediate)
+//
+// x is staged once per workgroup in LDS, zero-padded to a whole number of 64-lane vectors, and read back
+// as one ds_read_b128 per lane per chunk (conflict-free: consecutive lanes, consecutive 16 bytes).
+#pragma once
+#include "cats_device.h"
+
+namespace cats {
+
+enum RowsMode { kGate = 0, kGateUp = 1, kUp = 2, kGemv = 3 };
+
+struct RowsArgs {
+  const u32x4* x;        // (B, K) activations (K = row length of w)
+  const u32x4* w;        // (N, K) first weight: wgate (kGate, kGateUp), wup (kUp), W (kGemv)
+  const u32x4* w2;       // (N, K) wup for kGateUp
+  const void* a_in;      // kUp: (nb, N) gate activations in dtype
+  const uint8_t* flag_in;  // kUp: (nb, N)
+  void* a_out;           // kGate: (nb, N) dtype, optional
+  uint8_t* flag_out;     // kGate, kGateUp: (nb, N), optional
+  uint8_t* mask_out;     // kGate, kGateUp: ceil(N/8) bytes, bit j = OR over the batch of flag[b, j]; optional
+  float* z32_out;        // kGateUp: (nb, N) fp32, written for rows fetched from wup only; kUp: fp32 out, all rows
+  void* zt_out;          // kGateUp, kUp, kGemv: (nb, N) dtype, every row written (0 where inactive)
+  // compact list, kGate with nb == 1 only
+  uint32_t* arrive;      // zeroed counter; the last workgroup to finish builds the list and resets it
+  int64_t* idx_out;
+  void* vals_out;
+  int32_t* count_out;
+  int K;                 // row length in elements
+  int N;                 // number of rows
+  int nb;                // live batch rows (<= template B)
+  int nch;               // 64-lane vector chunks per row: ceil(K / (64 * VEC))
+  int row_vecs;          // K / VEC
+  float t;               // threshold, already rounded through dtype
+};
+
+// Dot products of R weight rows against the nb staged x rows.  acc[r][b] ends up wave-uniform.
+template <class DT, int B, int R, int CB, bool FULL, bool XLDS>
+__device__ __forceinline__ void rows_dot(const u32x4* __restrict__ w, const int (&row)[R], const bool (&on)[R],
+                                         const u32x4* xs, const u32x4* __restrict__ xg, const RowsArgs& p, int lane,
+                                         float (&acc)[R][B]) {
+#pragma unroll
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int b = 0; b < B; b++) acc[r][b] = 0.f;
+
+  // Loads are never predicated per lane: lanes past the end of a row re-read its last vector and meet a
+  // zero in x (the LDS copy of x is zero-padded to whole blocks of CB chunks), so a block of CB loads per
+  // row is issued back to back and stays in flight together.
+  const int vlast = p.row_vecs - 1;
+  const int nchp = (p.nch + CB - 1) / CB * CB;
+  for (int c0 = 0; c0 < p.nch; c0 += CB) {
+    u32x4 wv[R][CB];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      if (on[r]) {  // wave-uniform
+        const u32x4* wr = w + (size_t)row[r] * p.row_vecs;
+#pragma unroll
+        for (int cc = 0; cc < CB; cc++) {
+          const int v = (c0 + cc) * kWave + lane;
+          wv[r][cc] = load_stream(wr + (FULL ? v : min(v, vlast)));
+        }
+      }
+    }
+#pragma unroll
+    for (int cc = 0; cc < CB; cc++) {
+      const int v = (c0 + cc) * kWave + lane;
+#pragma unroll
+      for (int b = 0; b < B; b++) {
+        u32x4 xv;
+        if (XLDS) {
+          xv = xs[b * nchp * kWave + v];
+        } else {
+          xv = xg[(size_t)min(b, p.nb - 1) * p.row_vecs + min(v, vlast)];
+          if (!(b < p.nb && v < p.row_vecs)) xv = zero4();
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++)
+          if (on[r]) acc[r][b] = DT::dot(wv[r][cc], xv, acc[r][b]);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; r++)
+    if (on[r]) {
+#pragma unroll
+      for (int b = 0; b < B; b++) acc[r][b] = wave_sum(acc[r][b]);
+    }
+}
+
+template <class DT, int B, int R, int CB, bool FULL, int MODE, bool XLDS, int WAVES>
+__global__ __launch_bounds__(WAVES* kWave) void rows_kernel(RowsArgs p) {
+  typedef typename DT::st st;
+  extern __shared__ u32x4 xs[];  // [B][round_up(nch, CB) * 64] vectors (XLDS only)
+  __shared__ uint32_t s_maskbits;
+  __shared__ int s_last;
+  __shared__ int s_wtot[WAVES];
+
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  constexpr int kThreads = WAVES * kWave;
+  constexpr int kRowsPerBlock = WAVES * R;
+  static_assert(kRowsPerBlock % 8 == 0 && kRowsPerBlock <= 32, "mask bytes are assembled in one 32-bit LDS word");
+
+  if (XLDS) {
+    const int nchv = (p.nch + CB - 1) / CB * CB * kWave;  // padded vectors per x row
+    for (int i = threadIdx.x; i < B * nchv; i += kThreads) {
+      const int b = i / nchv, v = i - b * nchv;
+      u32x4 val = zero4();
+      if (b < p.nb && v < p.row_vecs) val = p.x[(size_t)b * p.row_vecs + v];
+      xs[i] = val;
+    }
+  }
+  if (threadIdx.x == 0) s_maskbits = 0u;
+  __syncthreads();
+
+  const int row0 = (blockIdx.x * WAVES + wave) * R;
+  int row[R];
+  bool on[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    row[r] = row0 + r < p.N ? row0 + r : p.N - 1;
+    on[r] = row0 + r < p.N;
+  }
+
+  float a[R][B];       // gate activation, rounded through dtype
+  bool act[R][B];      // per batch row flag
+  bool any[R];         // union over the batch
+
+  if (MODE == kUp) {
+    const st* ain = (const st*)p.a_in;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      any[r] = false;
+#pragma unroll
+      for (int b = 0; b < B; b++) {
+        act[r][b] = on[r] && b < p.nb && p.flag_in[(size_t)b * p.N + row[r]] != 0;
+        a[r][b] = act[r][b] ? DT::tof(ain[(size_t)b * p.N + row[r]]) : 0.f;
+        any[r] = any[r] || act[r][b];
+      }
+      // flags are per-lane loads of the same address; make the branch below provably wave-uniform
+      any[r] = __builtin_amdgcn_readfirstlane((int)any[r]) != 0;
+    }
+  } else {
+    float g[R][B];
+    rows_dot<DT, B, R, CB, FULL, XLDS>(p.w, row, on, xs, p.x, p, lane, g);
+    if (MODE == kGemv) {
+      if (lane == 0) {
+        st* out = (st*)p.zt_out;
+#pragma unroll
+        for (int r = 0; r < R; r++)
+          if (on[r]) {
+#pragma unroll
+            for (int b = 0; b < B; b++)
+              if (b < p.nb) out[(size_t)b * p.N + row[r]] = DT::fromf(g[r][b]);
+          }
+      }
+      return;
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      any[r] = false;
+#pragma unroll
+      for (int b = 0; b < B; b++) {
+        const float gr = DT::rnd(g[r][b]);
+        a[r][b] = DT::rnd(gr / (1.f + expf(-gr)));
+        act[r][b] = on[r] && b < p.nb && fabsf(a[r][b]) > p.t;
+        any[r] = any[r] || act[r][b];
+      }
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; r++)
+        if (on[r]) {
+#pragma unroll
+          for (int b = 0; b < B; b++)
+            if (b < p.nb) {
+              if (MODE == kGate && p.a_out) ((st*)p.a_out)[(size_t)b * p.N + row[r]] = DT::fromf(a[r][b]);
+              if (p.flag_out) p.flag_out[(size_t)b * p.N + row[r]] = act[r][b] ? 1 : 0;
+            }
+        }
+      if (p.mask_out) {
+        uint32_t bits = 0u;
+#pragma unroll
+        for (int r = 0; r < R; r++) bits |= (any[r] ? 1u : 0u) << (wave * R + r);
+        if (bits) atomicOr(&s_maskbits, bits);
+      }
+    }
+  }
+
+  if (MODE == kGateUp || MODE == kUp) {
+    float u[R][B];
+    rows_dot<DT, B, R, CB, FULL, XLDS>(MODE == kGateUp ? p.w2 : p.w, row, any, xs, p.x, p, lane, u);
+    if (lane == 0) {
+#pragma unroll
+      for (int r = 0; r < R; r++)
+        if (on[r]) {
+#pragma unroll
+          for (int b = 0; b < B; b++)
+            if (b < p.nb) {
+              const float z = act[r][b] ? DT::rnd(a[r][b] * DT::rnd(u[r][b])) : 0.f;
+              const size_t o = (size_t)b * p.N + row[r];
+              if (p.z32_out && (MODE == kUp || any[r])) p.z32_out[o] = z;
+              if (p.zt_out) ((st*)p.zt_out)[o] = DT::fromf(z);
+            }
+        }
+    }
+  }
+
+  if (MODE == kGate || MODE == kGateUp) {
+    if (p.mask_out) {
+      __syncthreads();
+      const int nbytes = (p.N + 7) >> 3;
+      if (threadIdx.x < kRowsPerBlock / 8) {
+        const int byte = blockIdx.x * (kRowsPerBlock / 8) + threadIdx.x;
+        if (byte < nbytes) p.mask_out[byte] = (uint8_t)(s_maskbits >> (8 * threadIdx.x));
+      }
+    }
+  }
+
+  if (MODE == kGate) {
+    if (p.idx_out == nullptr) return;
+    // Last workgroup to arrive turns the mask words into an ascending index list: one neuron per thread,
+    // wave ballot + mbcnt for the rank inside the wave, LDS prefix over the waves, running base per pass.
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const uint32_t prev = __hip_atomic_fetch_add(p.arrive, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = prev == gridDim.x - 1;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    const st* aall = (const st*)p.a_out;
+    int base = 0;
+    for (int j0 = 0; j0 < p.N; j0 += kThreads) {
+      const int j = j0 + threadIdx.x;
+      bool bit = false;
+      if (j < p.N) bit = (p.mask_out[j >> 3] >> (j & 7)) & 1;
+      const uint64_t ballot = __ballot(bit);
+      const int rank = ballot_rank(ballot);
+      if (lane == 0) s_wtot[wave] = __popcll(ballot);
+      __syncthreads();
+      int before = 0, total = 0;
+#pragma unroll
+      for (int w = 0; w < WAVES; w++) {
+        const int c = s_wtot[w];
+        if (w < wave) before += c;
+        total += c;
+      }
+      if (bit) {
+        const int o = base + before + rank;
+        p.idx_out[o] = j;
+        if (p.vals_out) ((st*)p.vals_out)[o] = aall[j];
+      }
+      base += total;
+      __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+      *p.count_out = base;
+      __hip_atomic_store(p.arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+}
+
+}  // namespace cats

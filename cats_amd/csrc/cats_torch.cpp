@@ -1,0 +1,353 @@
+// torch.ops.flash_gemv.* -- the op library the flash_gemv Python package loads.
+//
+// Same namespace, op names and positional signatures as the reference registration
+// (flash_gemv/csrc/fuse_gemv_cmp.cpp:87-102), so `torch.ops.flash_gemv.<op>(...)` call sites keep working.
+// Each op unpacks its tensors, checks device / dtype / contiguity / shapes, takes the current HIP stream
+// and a cached workspace, and calls one entry point of the C ABI in include/cats_gemv.h.  A non-zero
+// status becomes a c10::Error (the reference printf()s and exit()s: fuse_gemv_cmp_cuda.cu:2096-2097).
+#include <ATen/ATen.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/library.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+#include <utility>
+
+#include "cats_gemv.h"
+
+namespace {
+
+int dtype_code(const at::Tensor& t) {
+  switch (t.scalar_type()) {
+    case at::ScalarType::Half: return CATS_F16;
+    case at::ScalarType::BFloat16: return CATS_BF16;
+    case at::ScalarType::Float: return CATS_F32;
+    default: TORCH_CHECK(false, "flash_gemv: unsupported dtype ", t.scalar_type(), " (expected half, bfloat16 or float)");
+  }
+  return -1;
+}
+
+void check_status(int st, const char* op) {
+  TORCH_CHECK(st == CATS_OK, "flash_gemv.", op, ": ", cats_status_string(st));
+}
+
+void check_dev(const at::Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda(), "flash_gemv: ", name, " must be on the GPU");
+  TORCH_CHECK(t.is_contiguous(), "flash_gemv: ", name, " must be contiguous");
+}
+
+// Leading dims flattened into rows, as the reference does (fuse_gemv_cmp_cuda.cu:2339-2347).
+int batch_rows(const at::Tensor& input, const char* op) {
+  TORCH_CHECK(input.dim() == 2 || input.dim() == 3, "flash_gemv.", op, ": input must be (B, H) or (B, 1, H), got ", input.dim(), " dims");
+  const int64_t b = input.dim() == 3 ? input.size(0) * input.size(1) : input.size(0);
+  TORCH_CHECK(b >= 1 && b <= CATS_MAX_BATCH, "flash_gemv.", op, ": batch of ", b, " rows is not supported (1..", CATS_MAX_BATCH, ")");
+  return (int)b;
+}
+
+void check_weight(const at::Tensor& w, const at::Tensor& like, int64_t rows, int64_t cols, const char* name) {
+  check_dev(w, name);
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == rows && w.size(1) == cols, "flash_gemv: ", name, " must be (", rows, ", ", cols, "), got ", w.sizes());
+  TORCH_CHECK(w.scalar_type() == like.scalar_type(), "flash_gemv: ", name, " dtype ", w.scalar_type(), " differs from input dtype ", like.scalar_type());
+  TORCH_CHECK(w.device() == like.device(), "flash_gemv: ", name, " is on a different device than input");
+}
+
+struct Workspace {
+  at::Tensor buf;
+  size_t bytes = 0;
+};
+
+// One workspace per (device, stream, H, I): the carving of a workspace is tied to the layer shape.  It is
+// allocated and zero-filled (by a kernel on the calling stream) on the first call for a shape, so run one
+// call before capturing a HIP graph.
+Workspace& workspace(const at::Tensor& like, int B, int H, int I, hipStream_t stream) {
+  static std::mutex mu;
+  static std::map<std::tuple<int, void*, int, int>, Workspace> cache;
+  std::lock_guard<std::mutex> lock(mu);
+  Workspace& ws = cache[std::make_tuple((int)like.get_device(), (void*)stream, H, I)];
+  const size_t need = cats_workspace_bytes(B, H, I);
+  if (ws.bytes < need) {
+    ws.buf = at::empty({(int64_t)need}, like.options().dtype(at::kByte));
+    ws.bytes = need;
+    check_status(cats_workspace_init(ws.buf.data_ptr(), need, stream), "workspace_init");
+  }
+  return ws;
+}
+
+hipStream_t current_stream(const at::Tensor& t) { return c10::hip::getCurrentHIPStream(t.get_device()).stream(); }
+
+// ---- the 14 reference ops -----------------------------------------------------------------------------
+
+int64_t fuse_gemv_cmp(const at::Tensor& input, const at::Tensor& weight, at::Tensor& output, at::Tensor& idx,
+                      const double threshold) {
+  check_dev(input, "input");
+  const int B = batch_rows(input, "fuse_gemv_cmp");
+  TORCH_CHECK(B == 1, "flash_gemv.fuse_gemv_cmp: batch must be 1");
+  const int64_t H = input.size(-1), I = weight.size(0);
+  check_weight(weight, input, I, H, "weight");
+  check_dev(output, "output");
+  check_dev(idx, "idx");
+  TORCH_CHECK(output.scalar_type() == input.scalar_type() && output.numel() >= I, "flash_gemv.fuse_gemv_cmp: output must hold I values of the input dtype");
+  TORCH_CHECK(idx.scalar_type() == at::kLong && idx.numel() >= I, "flash_gemv.fuse_gemv_cmp: idx must be int64 with I entries");
+  hipStream_t s = current_stream(input);
+  Workspace& ws = workspace(input, 1, (int)H, (int)I, s);
+  int32_t* count = (int32_t*)((char*)ws.buf.data_ptr() + 768);
+  check_status(cats_gate_compact(input.data_ptr(), weight.data_ptr(), output.data_ptr(), idx.data_ptr<int64_t>(), count,
+                                 (int)H, (int)I, dtype_code(input), (float)threshold, ws.buf.data_ptr(), ws.bytes, s),
+               "fuse_gemv_cmp");
+  const int n = cats_read_count(count, s);
+  TORCH_CHECK(n >= 0, "flash_gemv.fuse_gemv_cmp: reading the count back failed");
+  return n;
+}
+
+void gate_flag_common(const at::Tensor& input, const at::Tensor& weight, at::Tensor& output, at::Tensor& flag,
+                      const double threshold, const char* op) {
+  check_dev(input, "input");
+  const int B = batch_rows(input, op);
+  const int64_t H = input.size(-1), I = weight.size(0);
+  check_weight(weight, input, I, H, "weight");
+  check_dev(output, "output");
+  check_dev(flag, "flag");
+  TORCH_CHECK(output.scalar_type() == input.scalar_type() && output.numel() == B * I, "flash_gemv.", op, ": output must be (B, I) of the input dtype");
+  TORCH_CHECK(flag.scalar_type() == at::kBool && flag.numel() == B * I, "flash_gemv.", op, ": flag must be bool with B*I entries");
+  check_status(cats_gate_flag(input.data_ptr(), weight.data_ptr(), output.data_ptr(), (uint8_t*)flag.data_ptr(), B, (int)H,
+                              (int)I, dtype_code(input), (float)threshold, current_stream(input)),
+               op);
+}
+
+void fuse_gemv_flag(const at::Tensor& input, const at::Tensor& weight, at::Tensor& output, at::Tensor& flag, const double threshold) {
+  gate_flag_common(input, weight, output, flag, threshold, "fuse_gemv_flag");
+}
+void fuse_gemv_flag_batch(const at::Tensor& input, const at::Tensor& weight, at::Tensor& output, at::Tensor& flag, const double threshold) {
+  gate_flag_common(input, weight, output, flag, threshold, "fuse_gemv_flag_batch");
+}
+void fuse_gemv_flag_local(const at::Tensor& input, const at::Tensor& weight, at::Tensor& output, at::Tensor& flag, const double threshold) {
+  gate_flag_common(input, weight, output, flag, threshold, "fuse_gemv_flag_local");
+}
+
+void fuse_gemv_flag_gemv(const at::Tensor& input, const at::Tensor& wgate, const at::Tensor& wup, at::Tensor& output,
+                         at::Tensor& flag, const double threshold) {
+  check_dev(input, "input");
+  const int B = batch_rows(input, "fuse_gemv_flag_gemv");
+  const int64_t H = input.size(-1), I = wgate.size(0);
+  check_weight(wgate, input, I, H, "wgate");
+  check_weight(wup, input, I, H, "wup");
+  check_dev(output, "output");
+  check_dev(flag, "flag");
+  TORCH_CHECK(output.scalar_type() == input.scalar_type() && output.numel() == B * I, "flash_gemv.fuse_gemv_flag_gemv: output must be (B, I) of the input dtype");
+  TORCH_CHECK(flag.scalar_type() == at::kBool && flag.numel() == B * I, "flash_gemv.fuse_gemv_flag_gemv: flag must be bool with B*I entries");
+  check_status(cats_gate_up(input.data_ptr(), wgate.data_ptr(), wup.data_ptr(), output.data_ptr(), (uint8_t*)flag.data_ptr(), B,
+                            (int)H, (int)I, dtype_code(input), (float)threshold, current_stream(input)),
+               "fuse_gemv_flag_gemv");
+}
+
+// Whole MLP, neuron-major down weights, fp32 accumulate into `output`.
+void mlp_f32_accumulate(const at::Tensor& input, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown,
+                        at::Tensor& output, at::Tensor* flag, const double threshold, const char* op) {
+  check_dev(input, "input");
+  const int B = batch_rows(input, op);
+  const int64_t H = input.size(-1), I = wgate.size(0);
+  check_weight(wgate, input, I, H, "wgate");
+  check_weight(wup, input, I, H, "wup");
+  check_weight(wdown, input, I, H, "wdown (neuron-major)");
+  check_dev(output, "output");
+  TORCH_CHECK(output.scalar_type() == at::kFloat && output.numel() == B * H, "flash_gemv.", op, ": output must be float32 with B*H entries");
+  uint8_t* fp = nullptr;
+  if (flag) {
+    check_dev(*flag, "flag");
+    TORCH_CHECK(flag->scalar_type() == at::kBool && flag->numel() == B * I, "flash_gemv.", op, ": flag must be bool with B*I entries");
+    fp = (uint8_t*)flag->data_ptr();
+  }
+  hipStream_t s = current_stream(input);
+  Workspace& ws = workspace(input, B, (int)H, (int)I, s);
+  check_status(cats_mlp(input.data_ptr(), wgate.data_ptr(), wup.data_ptr(), wdown.data_ptr(), nullptr, output.data_ptr<float>(), fp,
+                        nullptr, B, (int)H, (int)I, dtype_code(input), (float)threshold, ws.buf.data_ptr(), ws.bytes, s),
+               op);
+}
+
+void fuse_gemv_flag_gemv_gemv(const at::Tensor& input, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown,
+                              at::Tensor& output, at::Tensor& flag, const double threshold) {
+  mlp_f32_accumulate(input, wgate, wup, wdown, output, &flag, threshold, "fuse_gemv_flag_gemv_gemv");
+}
+void fuse_gemv_gemv_gemv(const at::Tensor& input, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown,
+                         at::Tensor& output, const double threshold) {
+  mlp_f32_accumulate(input, wgate, wup, wdown, output, nullptr, threshold, "fuse_gemv_gemv_gemv");
+}
+void flag_gemv_gemv_atomic(const at::Tensor& input, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown,
+                           at::Tensor& output, const double threshold) {
+  mlp_f32_accumulate(input, wgate, wup, wdown, output, nullptr, threshold, "flag_gemv_gemv_atomic");
+}
+
+void fuse_flag_gemv_local(const at::Tensor& input, const at::Tensor& weight, at::Tensor& output, at::Tensor& flag) {
+  check_dev(input, "input");
+  const int B = batch_rows(input, "fuse_flag_gemv_local");
+  const int64_t H = input.size(-1), I = weight.size(0);
+  check_weight(weight, input, I, H, "weight");
+  check_dev(output, "output");
+  check_dev(flag, "flag");
+  TORCH_CHECK(output.scalar_type() == input.scalar_type() && output.numel() == B * I, "flash_gemv.fuse_flag_gemv_local: output must be (B, I) of the input dtype");
+  TORCH_CHECK(flag.scalar_type() == at::kBool && flag.numel() == B * I, "flash_gemv.fuse_flag_gemv_local: flag must be bool with B*I entries");
+  check_status(cats_up_flag(input.data_ptr(), weight.data_ptr(), output.data_ptr(), (const uint8_t*)flag.data_ptr(), output.data_ptr(), 0,
+                            B, (int)H, (int)I, dtype_code(input), current_stream(input)),
+               "fuse_flag_gemv_local");
+}
+
+void atomic_gemv(const at::Tensor& input, const at::Tensor& weight, at::Tensor& output, at::Tensor& flag) {
+  check_dev(input, "input");
+  const int B = batch_rows(input, "atomic_gemv");
+  const int64_t I = input.size(-1), H = weight.size(1);
+  check_weight(weight, input, I, H, "weight (neuron-major)");
+  check_dev(output, "output");
+  check_dev(flag, "flag");
+  TORCH_CHECK(output.scalar_type() == at::kFloat && output.numel() == B * H, "flash_gemv.atomic_gemv: output must be float32 with B*H entries");
+  TORCH_CHECK(flag.scalar_type() == at::kBool && flag.numel() == B * I, "flash_gemv.atomic_gemv: flag must be bool with B*I entries");
+  hipStream_t s = current_stream(input);
+  Workspace& ws = workspace(input, B, (int)H, (int)I, s);
+  check_status(cats_down_flag(input.data_ptr(), weight.data_ptr(), (const uint8_t*)flag.data_ptr(), output.data_ptr<float>(), nullptr, B,
+                              (int)H, (int)I, dtype_code(input), ws.buf.data_ptr(), ws.bytes, s),
+               "atomic_gemv");
+}
+
+void mlp_rowmajor(const at::Tensor& input, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown, at::Tensor& output,
+                  const double threshold, const char* op) {
+  check_dev(input, "input");
+  const int B = batch_rows(input, op);
+  const int64_t H = input.size(-1), I = wgate.size(0);
+  check_weight(wgate, input, I, H, "wgate");
+  check_weight(wup, input, I, H, "wup");
+  check_weight(wdown, input, H, I, "wdown");
+  check_dev(output, "output");
+  TORCH_CHECK(output.scalar_type() == input.scalar_type() && output.numel() == B * H, "flash_gemv.", op, ": output must be (B, H) of the input dtype");
+  hipStream_t s = current_stream(input);
+  Workspace& ws = workspace(input, B, (int)H, (int)I, s);
+  check_status(cats_mlp_rowmajor_down(input.data_ptr(), wgate.data_ptr(), wup.data_ptr(), wdown.data_ptr(), output.data_ptr(), B, (int)H,
+                                      (int)I, dtype_code(input), (float)threshold, ws.buf.data_ptr(), ws.bytes, s),
+               op);
+}
+
+void flag_gemv_gemv(const at::Tensor& input, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown, at::Tensor& output,
+                    const double threshold) {
+  mlp_rowmajor(input, wgate, wup, wdown, output, threshold, "flag_gemv_gemv");
+}
+
+at::Tensor inner_common(const at::Tensor& input, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown,
+                        const double threshold, at::ScalarType want, const char* op) {
+  TORCH_CHECK(input.scalar_type() == want, "flash_gemv.", op, ": input must be ", want, ", got ", input.scalar_type());
+  at::Tensor output = at::empty(input.sizes(), input.options());
+  mlp_rowmajor(input, wgate, wup, wdown, output, threshold, op);
+  return output;
+}
+at::Tensor flag_gemv_gemv_inner(const at::Tensor& input, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown, const double threshold) {
+  return inner_common(input, wgate, wup, wdown, threshold, at::kHalf, "flag_gemv_gemv_inner");
+}
+at::Tensor flag_gemv_gemv_inner_fp32(const at::Tensor& input, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown, const double threshold) {
+  return inner_common(input, wgate, wup, wdown, threshold, at::kFloat, "flag_gemv_gemv_inner_fp32");
+}
+at::Tensor flag_gemv_gemv_inner_bf16(const at::Tensor& input, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown, const double threshold) {
+  return inner_common(input, wgate, wup, wdown, threshold, at::kBFloat16, "flag_gemv_gemv_inner_bf16");
+}
+
+// ---- ops behind the Python composites (the reference runs Triton there: flash_gemv/flash_gemv/kernels.py) ---
+
+// gather_gemv_elemul_flag_3d: x (B,1,H), x_1 (B,1,I), wup (I,H), flags (B,1,I) bool -> (B,1,I) in x.dtype
+at::Tensor cats_up_flag_op(const at::Tensor& x, const at::Tensor& x_1, const at::Tensor& wup, const at::Tensor& flags) {
+  check_dev(x, "x");
+  const int B = batch_rows(x, "cats_up_flag");
+  const int64_t H = x.size(-1), I = wup.size(0);
+  check_weight(wup, x, I, H, "wup");
+  check_dev(x_1, "x_1");
+  check_dev(flags, "flags");
+  TORCH_CHECK(x_1.scalar_type() == x.scalar_type() && x_1.numel() == B * I, "flash_gemv.cats_up_flag: x_1 must be (B, I) of x's dtype");
+  TORCH_CHECK(flags.scalar_type() == at::kBool && flags.numel() == B * I, "flash_gemv.cats_up_flag: flags must be bool with B*I entries");
+  at::Tensor out = at::empty_like(x_1);
+  check_status(cats_up_flag(x.data_ptr(), wup.data_ptr(), x_1.data_ptr(), (const uint8_t*)flags.data_ptr(), out.data_ptr(), 0, B, (int)H,
+                            (int)I, dtype_code(x), current_stream(x)),
+               "cats_up_flag");
+  return out;
+}
+
+// gather_transposed_gemv_flag_3d: x (B,1,I), weight (I,H) neuron-major, flags (B,1,I) -> (B,1,H) in weight.dtype
+at::Tensor cats_down_flag_op(const at::Tensor& x, const at::Tensor& weight, const at::Tensor& flags) {
+  check_dev(x, "x");
+  const int B = batch_rows(x, "cats_down_flag");
+  const int64_t I = weight.size(0), H = weight.size(1);
+  check_weight(weight, x, I, H, "weight (neuron-major)");
+  check_dev(flags, "flags");
+  TORCH_CHECK(x.size(-1) == I, "flash_gemv.cats_down_flag: x must have I columns");
+  TORCH_CHECK(flags.scalar_type() == at::kBool && flags.numel() == B * I, "flash_gemv.cats_down_flag: flags must be bool with B*I entries");
+  std::vector<int64_t> shape(x.sizes().begin(), x.sizes().end());
+  shape.back() = H;
+  at::Tensor out = at::empty(shape, weight.options());
+  hipStream_t s = current_stream(x);
+  Workspace& ws = workspace(x, B, (int)H, (int)I, s);
+  check_status(cats_down_flag(x.data_ptr(), weight.data_ptr(), (const uint8_t*)flags.data_ptr(), nullptr, out.data_ptr(), B, (int)H, (int)I,
+                              dtype_code(x), ws.buf.data_ptr(), ws.bytes, s),
+               "cats_down_flag");
+  return out;
+}
+
+// Whole CATS MLP in two launches: x (B,1,H) or (B,H); wgate, wup, wdown_t all (I,H).  Returns x-shaped y.
+at::Tensor cats_mlp_op(const at::Tensor& x, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown_t, const double threshold) {
+  check_dev(x, "x");
+  const int B = batch_rows(x, "cats_mlp");
+  const int64_t H = x.size(-1), I = wgate.size(0);
+  check_weight(wgate, x, I, H, "wgate");
+  check_weight(wup, x, I, H, "wup");
+  check_weight(wdown_t, x, I, H, "wdown_t (neuron-major)");
+  at::Tensor out = at::empty_like(x);
+  hipStream_t s = current_stream(x);
+  Workspace& ws = workspace(x, B, (int)H, (int)I, s);
+  check_status(cats_mlp(x.data_ptr(), wgate.data_ptr(), wup.data_ptr(), wdown_t.data_ptr(), out.data_ptr(), nullptr, nullptr, nullptr, B, (int)H,
+                        (int)I, dtype_code(x), (float)threshold, ws.buf.data_ptr(), ws.bytes, s),
+               "cats_mlp");
+  return out;
+}
+
+// Same, also returning the per-row flags (B*I bool) and the number of neurons fetched (int32 scalar tensor).
+std::tuple<at::Tensor, at::Tensor, at::Tensor> cats_mlp_stats_op(const at::Tensor& x, const at::Tensor& wgate, const at::Tensor& wup,
+                                                                 const at::Tensor& wdown_t, const double threshold) {
+  check_dev(x, "x");
+  const int B = batch_rows(x, "cats_mlp_stats");
+  const int64_t H = x.size(-1), I = wgate.size(0);
+  check_weight(wgate, x, I, H, "wgate");
+  check_weight(wup, x, I, H, "wup");
+  check_weight(wdown_t, x, I, H, "wdown_t (neuron-major)");
+  at::Tensor out = at::empty_like(x);
+  at::Tensor flags = at::empty({B, I}, x.options().dtype(at::kBool));
+  at::Tensor count = at::empty({}, x.options().dtype(at::kInt));
+  hipStream_t s = current_stream(x);
+  Workspace& ws = workspace(x, B, (int)H, (int)I, s);
+  check_status(cats_mlp(x.data_ptr(), wgate.data_ptr(), wup.data_ptr(), wdown_t.data_ptr(), out.data_ptr(), nullptr, (uint8_t*)flags.data_ptr(),
+                        count.data_ptr<int32_t>(), B, (int)H, (int)I, dtype_code(x), (float)threshold, ws.buf.data_ptr(), ws.bytes, s),
+               "cats_mlp_stats");
+  return {out, flags, count};
+}
+
+void cats_set_tuning_op(int64_t gate_variant, int64_t down_groups, int64_t down_block) {
+  cats_set_tuning((int)gate_variant, (int)down_groups, (int)down_block);
+}
+
+}  // namespace
+
+TORCH_LIBRARY(flash_gemv, m) {
+  m.def("fuse_gemv_cmp", fuse_gemv_cmp);
+  m.def("fuse_gemv_flag", fuse_gemv_flag);
+  m.def("fuse_gemv_flag_gemv", fuse_gemv_flag_gemv);
+  m.def("fuse_gemv_flag_gemv_gemv", fuse_gemv_flag_gemv_gemv);
+  m.def("fuse_gemv_gemv_gemv", fuse_gemv_gemv_gemv);
+  m.def("fuse_gemv_flag_batch", fuse_gemv_flag_batch);
+  m.def("fuse_gemv_flag_local", fuse_gemv_flag_local);
+  m.def("fuse_flag_gemv_local", fuse_flag_gemv_local);
+  m.def("atomic_gemv", atomic_gemv);
+  m.def("flag_gemv_gemv_atomic", flag_gemv_gemv_atomic);
+  m.def("flag_gemv_gemv", flag_gemv_gemv);
+  m.def("flag_gemv_gemv_inner", flag_gemv_gemv_inner);
+  m.def("flag_gemv_gemv_inner_fp32", flag_gemv_gemv_inner_fp32);
+  m.def("flag_gemv_gemv_inner_bf16", flag_gemv_gemv_inner_bf16);
+  // HIP replacements for the Triton wrappers and the fused two-launch MLP
+  m.def("cats_up_flag", cats_up_flag_op);
+  m.def("cats_down_flag", cats_down_flag_op);
+  m.def("cats_mlp", cats_mlp_op);
+  m.def("cats_mlp_stats", cats_mlp_stats_op);
+  m.def("cats_set_tuning", cats_set_tuning_op);
+}

@@ -1,0 +1,139 @@
+/*
+ * cats_gemv.h -- C ABI of the gfx950 CATS sparse-MLP decode kernels.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream and returns a
+ * cats_status_t.  Nothing here allocates, frees or synchronises (cats_read_count is the one
+ * documented exception: it has to hand a device counter back to the host).  All launches go
+ * to the stream that is passed in.  The entry points are what a `TORCH_LIBRARY(flash_gemv, m)`
+ * shim, a ctypes loader or any other FFI binds; each one names the reference interface it
+ * stands in for (paths relative to the CATS tree).
+ *
+ * Conventions
+ *   B      rows of the activation matrix (batch * seq, decode => seq == 1); 1 <= B <= CATS_MAX_BATCH
+ *   H      hidden size, I intermediate size
+ *   dtype  cats_dtype_t; x, weights and dtype-typed outputs all share it
+ *   x        (B, H)  row-major
+ *   wgate    (I, H)  row-major  (nn.Linear layout: one row per neuron)
+ *   wup      (I, H)  row-major
+ *   wdown_t  (I, H)  row-major, "neuron-major": row j is column j of the HF down_proj.weight
+ *   wdown    (H, I)  row-major  (HF nn.Linear layout)
+ *   flag     (B, I)  one byte per entry, 0 or 1 (torch.bool storage)
+ *   Rows must be 16-byte aligned: H * sizeof(dtype) % 16 == 0 and all base pointers 16-byte
+ *   aligned (I * sizeof(dtype) % 16 == 0 as well where I is a row length: wdown, a, z).
+ *
+ * Activation and mask rule (experiments/models/sparse_silu/ugly_utils.py:895-899,
+ * flash_gemv/flash_gemv/__init__.py:41,46):
+ *   g  = round_dtype(sum_k x[b,k] * wgate[j,k])        fp32 accumulation
+ *   a  = round_dtype(g / (1 + exp(-g)))                SiLU evaluated in fp32
+ *   active(b,j)  <=>  |a| > round_dtype(threshold)     strict, compared on the stored value
+ *   z  = active ? round_dtype(a * round_dtype(sum_k x[b,k] * wup[j,k])) : 0
+ *   y  = round_dtype(sum_j z[b,j] * wdown_t[j,:])      fp32 accumulation
+ * A weight row of wup / wdown_t is fetched only if some row b of the batch has it active.
+ */
+#ifndef CATS_GEMV_H
+#define CATS_GEMV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { CATS_F16 = 0, CATS_BF16 = 1, CATS_F32 = 2 } cats_dtype_t;
+
+typedef enum {
+  CATS_OK = 0,
+  CATS_ERR_DTYPE = 1,      /* dtype is not a cats_dtype_t */
+  CATS_ERR_SHAPE = 2,      /* non-positive or unsupported H / I */
+  CATS_ERR_ALIGN = 3,      /* a pointer or row pitch is not 16-byte aligned */
+  CATS_ERR_BATCH = 4,      /* B outside 1..CATS_MAX_BATCH */
+  CATS_ERR_NULL = 5,       /* a required pointer is NULL */
+  CATS_ERR_WORKSPACE = 6,  /* workspace missing or smaller than cats_workspace_bytes() */
+  CATS_ERR_LAUNCH = 7      /* the HIP runtime refused a launch; hipGetLastError() has details */
+} cats_status_t;
+
+#define CATS_MAX_BATCH 8
+#define CATS_MAX_INTERMEDIATE 65536 /* sparse down kernel scans I/64 mask words in one block */
+
+/* Library identification / error text.  No reference counterpart (the reference printf()s and exit()s:
+ * flash_gemv/csrc/cuda/fuse_gemv_cmp_cuda.cu:25-33,2397-2400). */
+int cats_version(void);
+const char* cats_status_string(int status);
+
+/* Workspace: scratch for the mask words, the fp32 intermediate z, the fp32 output accumulator and a few
+ * counters.  Replaces the per-call cudaMalloc/cudaFree pairs of the reference
+ * (fuse_gemv_cmp_cuda.cu:2351-2354,2402-2403).  The caller allocates cats_workspace_bytes() once (256-byte
+ * aligned), runs cats_workspace_init() once (it zero-fills with a kernel), and then passes the same buffer to
+ * every call; each call leaves the parts that must start at zero zeroed again.  The size and the carving
+ * depend on (H, I) only (B is checked, every region holds CATS_MAX_BATCH rows), so one workspace serves every
+ * batch size of one layer shape; for another (H, I) use another workspace or initialise again.  One workspace
+ * serves one stream at a time. */
+size_t cats_workspace_bytes(int B, int H, int I);
+int cats_workspace_init(void* ws, size_t ws_bytes, void* stream);
+
+/* Fused gate GEMV + SiLU + |a| > t.  Writes a (B,I) in dtype and/or flag (B,I) bytes; either may be NULL.
+ * Replaces fuse_gemv_flag_local / fuse_gemv_flag / fuse_gemv_flag_batch
+ * (flash_gemv/flash_gemv/flash_gemv.py:6-7,18-22; fuse_gemv_cmp_cuda.cu:1292-1486,2083-2117). */
+int cats_gate_flag(const void* x, const void* wgate, void* a_out, uint8_t* flag_out,
+                   int B, int H, int I, int dtype, float threshold, void* stream);
+
+/* Same gate pass, B == 1, that also emits the compact active set: idx_out[0..count) ascending neuron
+ * indices (int64), vals_out[0..count) the matching activations in dtype, *count_out (device int32) the
+ * count.  The list is built by the last workgroup to finish, with wave ballots and a prefix sum.
+ * Replaces fuse_gemv_cmp (flash_gemv.py:3-4; fuse_gemv_cmp_cuda.cu:43-88,1962-1977), whose list is in
+ * atomic arrival order and whose count lives in a process-global managed int. */
+int cats_gate_compact(const void* x, const void* wgate, void* vals_out, int64_t* idx_out, int32_t* count_out,
+                      int H, int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream);
+
+/* Blocking helper for the call above: waits for the stream and returns *count_dev (or -1 on error). */
+int cats_read_count(const int32_t* count_dev, void* stream);
+
+/* Sparse up projection over a flag array.  out[b,j] = flag[b,j] ? a[b,j] * (x[b,:] . wup[j,:]) : 0.
+ * Row j of wup is fetched iff any flag[b,j] is set.  a and out are (B,I); out may alias a (in place).
+ * out_is_f32 != 0 writes fp32 instead of dtype.
+ * Replaces fuse_flag_gemv_local (flash_gemv.py:24-25; fuse_gemv_cmp_cuda.cu:1507-1722,2123-2156) and the
+ * Triton gather_gemv_elemul_flag_3d (flash_gemv/flash_gemv/kernels.py:69-254). */
+int cats_up_flag(const void* x, const void* wup, const void* a, const uint8_t* flag, void* out, int out_is_f32,
+                 int B, int H, int I, int dtype, void* stream);
+
+/* Sparse down projection over neuron-major weights.  y[b,:] += sum_{j: any flag[.,j]} z[b,j] * wdown_t[j,:].
+ * z is (B,I) in dtype.  Two output modes:
+ *   y_f32 != NULL : fp32 atomics straight into the caller's (B,H) buffer, which the caller zeroed (or wants
+ *                   accumulated into) -- atomic_gemv (flash_gemv.py:27-28; fuse_gemv_cmp_cuda.cu:1724-1783,2162-2194);
+ *   y_out != NULL : (B,H) in dtype, zero-initialised and rounded inside the call -- the Triton
+ *                   gather_transposed_gemv_flag_3d (kernels.py:324-462).
+ * Exactly one of y_f32 / y_out must be non-NULL.  Needs a workspace. */
+int cats_down_flag(const void* z, const void* wdown_t, const uint8_t* flag, float* y_f32, void* y_out,
+                   int B, int H, int I, int dtype, void* ws, size_t ws_bytes, void* stream);
+
+/* Gate + sparse up in one pass: out[b,j] = active ? round(a * up) : 0 in dtype, flag_out optional.
+ * Replaces fuse_gemv_flag_gemv (flash_gemv.py:9-10; fuse_gemv_cmp_cuda.cu:715-784,2006-2022). */
+int cats_gate_up(const void* x, const void* wgate, const void* wup, void* out, uint8_t* flag_out,
+                 int B, int H, int I, int dtype, float threshold, void* stream);
+
+/* Whole CATS MLP with neuron-major down weights: two launches (gate+up, sparse down).
+ *   y_out != NULL : (B,H) in dtype;  y_f32 != NULL : fp32 accumulate into the caller's pre-zeroed (B,H).
+ * flag_out (B,I) optional.  count_out (device int32, optional) receives the number of neurons fetched
+ * (union over the batch).
+ * Replaces flag_gemv_gemv_atomic, fuse_gemv_gemv_gemv, fuse_gemv_flag_gemv_gemv (flash_gemv.py:12-16,30-31;
+ * fuse_gemv_cmp_cuda.cu:786-1244,2196-2253) and the composite gemv_gemv_triton / flag_gemv_gemv_triton
+ * (flash_gemv/flash_gemv/__init__.py:38-48). */
+int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, float* y_f32,
+             uint8_t* flag_out, int32_t* count_out, int B, int H, int I, int dtype, float threshold,
+             void* ws, size_t ws_bytes, void* stream);
+
+/* Whole CATS MLP with the HF (H,I) down weight: gate+up, then a dense row-major GEMV over the zero-filled
+ * intermediate (all of wdown is read, as in the reference).
+ * Replaces flag_gemv_gemv and flag_gemv_gemv_inner{,_fp32,_bf16} (flash_gemv.py:33-43;
+ * fuse_gemv_cmp_cuda.cu:2255-2560). */
+int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out,
+                           int B, int H, int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream);
+
+/* Launch-shape knobs for experiments and profiling; 0 keeps the built-in choice.  Not in the reference. */
+int cats_set_tuning(int gate_variant, int down_groups, int down_block);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CATS_GEMV_H */

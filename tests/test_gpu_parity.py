@@ -1,0 +1,306 @@
+"""GPU parity: the HIP kernels, called through the C ABI (cats_amd.capi -> libcats_gemv.so), against the CPU
+oracle on the same seeded inputs.
+
+Bar: masks bit-exact against the reference rule |a| > t evaluated on identical gate values (the kernel's own
+stored activations); outputs within rtol 1e-2 / atol 2e-3 (fp16, bf16) and 1e-5 (fp32) of the dense-masked MLP.
+"""
+import math
+
+import pytest
+import torch
+
+from tests.util import A_TOL, TOL, calibrate, dev, make_mlp
+
+pytestmark = pytest.mark.gpu
+
+capi = None
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _load():
+    global capi
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    from cats_amd import capi as _capi
+
+    _capi.lib()
+    capi = _capi
+
+
+def _ws(B, H, I):
+    return capi.Workspace(B, H, I)
+
+
+def close(got, want, dtype):
+    """The parity tolerance.  atol is stated for outputs of order one (the benchmark configurations); for the
+    reference's U(-0.5, 0.5) recipe, whose outputs reach the hundreds, it scales with the largest output."""
+    tol = dict(TOL[dtype])
+    tol["atol"] *= max(1.0, float(want.float().abs().max()))
+    torch.testing.assert_close(got.float(), want.float(), **tol)
+
+
+def check_mlp_case(oracle, m, t, *, tag, ws=None, expect_flip_free=False):
+    """Full set of parity checks for one (weights, x, threshold)."""
+    dtype = m["x"].dtype
+    B, H = m["x"].shape
+    I = m["wg"].shape[0]
+    print(f"[case] {tag} dtype={dtype} B={B} H={H} I={I} t={t}", flush=True)
+    d = dev(m)
+    ws = ws or _ws(B, H, I)
+
+    a, flag = capi.gate_flag(d["x"], d["wg"], t)
+    y, flag2, count = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
+    if (I * m["x"].element_size()) % 16 == 0:
+        y_rm = capi.mlp_rowmajor_down(d["x"], d["wg"], d["wu"], d["wd"], t, ws)
+    else:  # rows of the (H, I) down weight are not 16-byte aligned: rejected, not mis-read
+        with pytest.raises(capi.CatsError, match="aligned"):
+            capi.mlp_rowmajor_down(d["x"], d["wg"], d["wu"], d["wd"], t, ws)
+        y_rm = y
+    torch.cuda.synchronize()
+    a, flag, y, flag2, y_rm = a.cpu(), flag.cpu(), y.cpu(), flag2.cpu(), y_rm.cpu()
+
+    # 1. mask rule, bit-exact on identical gate values: torch's own comparison on the kernel's activations
+    want_flag = torch.abs(a) > t
+    assert torch.equal(flag, want_flag), f"{tag}: flag != (|a| > t) on the kernel's own a"
+    assert torch.equal(flag2, flag), f"{tag}: the fused MLP pass and the gate pass disagree on flags"
+    union = flag.any(dim=0)
+    assert int(count.item()) == int(union.sum()), f"{tag}: active count {int(count.item())} != {int(union.sum())}"
+    # the C oracle's rule on the same activations (independent of torch's scalar casting)
+    tr = oracle.c_round(dtype, t)
+    assert torch.equal(flag, a.float().abs() > tr)
+
+    # 2. activations vs the oracle's own gate stage
+    ref = oracle.c_mlp(m["x"], m["wg"], m["wu"], m["wd"], t)
+    a_tol = dict(A_TOL[dtype])
+    a_tol["atol"] *= max(1.0, float(ref["a"].float().abs().max()))  # same scaling rule as close()
+    torch.testing.assert_close(a.float(), ref["a"].float(), **a_tol)
+
+    # 3. mask vs the oracle's mask on ITS gate values: may differ only within rounding distance of t
+    flips = flag != ref["flag"]
+    nflip = int(flips.sum())
+    if nflip:
+        band = a_tol["atol"] + a_tol["rtol"] * abs(tr)
+        dist = (ref["a"].float().abs() - tr).abs()[flips]
+        assert float(dist.max()) <= band, f"{tag}: {nflip} mask flips, one {float(dist.max())} away from t (band {band})"
+    print(f"        active={int(union.sum())}/{I} flips_vs_oracle={nflip}", flush=True)
+    if expect_flip_free:
+        assert nflip == 0
+
+    # 4. output vs the dense-masked oracle on identical gate values (kernel's a and flags fed to the oracle)
+    ref_same = oracle.c_mlp(m["x"], m["wg"], m["wu"], m["wd"], t, a_in=a, flag_in=flag)
+    close(y, ref_same["y"], dtype)
+    close(y_rm, ref_same["y"], dtype)
+    # 5. and vs the fully independent oracle / the literal PyTorch formula when no flag flipped
+    if nflip == 0:
+        close(y, ref["y"], dtype)
+        if dtype == torch.float32:
+            y_t, _, dead = oracle.torch_cats_mlp(m["x"], m["wg"], m["wu"], m["wd"], t)
+            if torch.equal(~dead, flag):
+                close(y, y_t, dtype)
+    return dict(y=y, a=a, flag=flag)
+
+
+SMALL = [
+    # H, I, B, dtype
+    (64, 96, 1, torch.float16), (64, 96, 2, torch.bfloat16), (64, 96, 3, torch.float32),
+    (72, 100, 1, torch.float16),      # H not a multiple of 64 vectors, I not a multiple of 8
+    (520, 1000, 4, torch.float16), (512, 1024, 8, torch.bfloat16), (260, 333, 5, torch.float32),
+    (4096, 512, 1, torch.float16), (2048, 640, 2, torch.float32), (8192, 256, 1, torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("H,I,B,dtype", SMALL)
+@pytest.mark.parametrize("dist", ["normal", "uniform"])
+def test_small_shapes(oracle, H, I, B, dtype, dist):
+    m = make_mlp(H, I, B, dtype, seed=H * 7 + I + B, dist=dist)
+    scale = 1.0 if dist == "normal" else 1.0
+    a_abs = oracle.c_gate(m["x"], m["wg"], -1.0)[0].float().abs().flatten()
+    for q in (0.0, 0.5, 0.9):
+        t = -1.0 if q == 0.0 else float(torch.quantile(a_abs, q)) * scale
+        check_mlp_case(oracle, m, t, tag=f"small-{dist}-q{q}")
+
+
+def test_all_dead_and_all_active(oracle):
+    m = make_mlp(512, 768, 2, torch.float16, seed=5)
+    d = dev(m)
+    ws = _ws(2, 512, 768)
+    y = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], float("inf"), ws)
+    assert torch.count_nonzero(y) == 0
+    # a second call on the same workspace after an all-dead call must still be right (accumulator stays clean)
+    y = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], -1.0, ws)
+    dense = oracle.torch_dense_mlp(m["x"].float(), m["wg"].float(), m["wu"].float(), m["wd"].float())
+    torch.testing.assert_close(y.cpu().float(), dense, **TOL[torch.float16])
+
+
+def test_single_active_neuron_is_exact(oracle):
+    """One live neuron: y = round(z_j * wdown_t[j, :]) -- a single product per column, bit-checkable."""
+    for dtype in (torch.float16, torch.bfloat16, torch.float32):
+        m = make_mlp(256, 384, 1, dtype, seed=11)
+        d = dev(m)
+        a, _ = capi.gate_flag(d["x"], d["wg"], -1.0)
+        mags = a.float().abs().flatten().sort(descending=True).values
+        assert mags[0] > mags[1]
+        t = float((mags[0] + mags[1]) / 2)
+        ws = _ws(1, 256, 384)
+        y, flag, count = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
+        assert int(count.item()) == 1 and int(flag.sum()) == 1
+        j = int(flag.flatten().nonzero()[0])
+        z = capi.gate_up(d["x"], d["wg"], d["wu"], t)[0][0, j]
+        want = (z.float() * d["wdt"][j].float()).to(dtype)
+        assert torch.equal(y[0], want), f"{dtype}: single-neuron output is not the exact product"
+
+
+def test_workspace_reuse_and_repeatability(oracle):
+    """Back-to-back calls on one workspace (different thresholds and batch sizes) do not contaminate each other."""
+    H, I = 1024, 2048
+    ws = _ws(8, H, I)
+    outs = {}
+    for rep in range(2):
+        for B, q in ((8, 0.5), (1, 0.9), (4, 0.0), (2, 0.7)):
+            m = make_mlp(H, I, B, torch.float16, seed=100 + B)
+            a_abs = oracle.c_gate(m["x"], m["wg"], -1.0)[0].float().abs().flatten()
+            t = -1.0 if q == 0.0 else float(torch.quantile(a_abs, q))
+            d = dev(m)
+            y = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws).cpu()
+            ref = oracle.c_mlp(m["x"], m["wg"], m["wu"], m["wd"], t)
+            torch.testing.assert_close(y.float(), ref["y"].float(), **TOL[torch.float16])
+            if rep == 0:
+                outs[B] = y
+            else:
+                torch.testing.assert_close(y.float(), outs[B].float(), **TOL[torch.float16])
+
+
+def test_batch_rows_are_independent(oracle):
+    """Row b of a batched call equals the single-row call on x[b] (union gathering must not leak between rows)."""
+    H, I, B = 1024, 1536, 4
+    m = make_mlp(H, I, B, torch.float16, seed=21, corr=0.5)
+    t = calibrate(m["wg"], [0.5])[0]
+    d = dev(m)
+    ws = _ws(B, H, I)
+    yb, fb, _ = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
+    for b in range(B):
+        y1, f1, _ = capi.mlp(d["x"][b:b + 1].contiguous(), d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
+        assert torch.equal(f1[0], fb[b])
+        torch.testing.assert_close(y1[0].float(), yb[b].float(), **TOL[torch.float16])
+
+
+def test_gate_compact_list(oracle):
+    for (H, I, dtype) in ((64, 96, torch.float16), (512, 1000, torch.bfloat16), (4096, 2048, torch.float16), (256, 300, torch.float32)):
+        m = make_mlp(H, I, 1, dtype, seed=31)
+        d = dev(m)
+        ws = _ws(1, H, I)
+        for q in (0.0, 0.5, 0.95, 1.1):
+            a_ref, _ = capi.gate_flag(d["x"], d["wg"], -1.0)
+            mags = a_ref.float().abs().flatten()
+            t = -1.0 if q == 0.0 else (float("inf") if q > 1 else float(torch.quantile(mags, q)))
+            for _ in range(2):  # twice: the arrival counter must reset itself
+                vals, idx, n = capi.gate_compact(d["x"], d["wg"], t, ws)
+                a, flag = capi.gate_flag(d["x"], d["wg"], t)
+                want_idx, want_n = oracle.c_compact(flag[0])
+                assert n == want_n == int(flag.sum())
+                assert torch.equal(idx[:n].cpu(), want_idx), "index list is not ascending nonzero(mask)"
+                assert torch.equal(vals[:n].cpu(), a[0].cpu()[want_idx])
+
+
+def test_sparse_up_and_down_ops(oracle):
+    """The stand-alone flag-driven up / down entry points against the oracle's restatement of the Triton pair."""
+    for (H, I, B, dtype) in ((512, 1024, 1, torch.float16), (1024, 1000, 3, torch.bfloat16), (256, 512, 2, torch.float32), (4096, 1024, 4, torch.float16)):
+        m = make_mlp(H, I, B, dtype, seed=41, corr=0.5)
+        d = dev(m)
+        t = calibrate(m["wg"], [0.6])[0]
+        a, flag = capi.gate_flag(d["x"], d["wg"], t)
+        z32 = capi.up_flag(d["x"], d["wu"], a, flag, out_f32=True)
+        zt = capi.up_flag(d["x"], d["wu"], a, flag, out_f32=False)
+        want_z = oracle.c_sparse_up(m["x"], m["wu"], a, flag)
+        torch.testing.assert_close(z32.cpu(), want_z, **TOL[dtype])
+        torch.testing.assert_close(zt.cpu().float(), want_z, **TOL[dtype])
+        assert torch.count_nonzero(zt[~flag]) == 0
+        ws = _ws(B, H, I)
+        y = capi.down_flag(zt, d["wdt"], flag, ws)
+        want_y = oracle.c_sparse_down(zt, m["wdt"], flag)
+        torch.testing.assert_close(y.cpu().float(), want_y, **TOL[dtype])
+        acc = torch.ones(B, H, dtype=torch.float32, device="cuda")   # accumulate mode: adds onto what is there
+        capi.down_flag(zt, d["wdt"], flag, ws, accumulate_into=acc)
+        tol = dict(TOL[dtype]); tol["atol"] = max(tol["atol"], 1e-4)
+        torch.testing.assert_close(acc.cpu() - 1.0, want_y, **tol)
+        gu, gflag = capi.gate_up(d["x"], d["wg"], d["wu"], t)
+        assert torch.equal(gflag, flag)
+        torch.testing.assert_close(gu.cpu().float(), want_z, **TOL[dtype])
+
+
+# ---- the benchmark configurations at full size ---------------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def llama_fp16():
+    return make_mlp(4096, 11008, 1, torch.float16, seed=0)
+
+
+def test_config2_llama_fp16_sweep(oracle, llama_fp16):
+    m = llama_fp16
+    ts = calibrate(m["wg"], [0.0, 0.3, 0.5, 0.7, 0.9])
+    ws = _ws(1, 4096, 11008)
+    for s, t in zip([0.0, 0.3, 0.5, 0.7, 0.9], ts):
+        r = check_mlp_case(oracle, m, t, tag=f"llama-fp16-s{s}", ws=ws)
+        got = 1.0 - float(r["flag"].float().mean())
+        assert abs(got - s) < 0.03, f"sparsity {got} far from target {s}"
+
+
+def test_config2_all_active_matches_dense_gemv(oracle, llama_fp16):
+    """0 % sparsity reduces to the dense SwiGLU MLP = three library GEMVs (rocBLAS through torch, on the GPU)."""
+    d = dev(llama_fp16)
+    ws = _ws(1, 4096, 11008)
+    y = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], -1.0, ws)
+    dense = oracle.torch_dense_mlp(d["x"], d["wg"], d["wu"], d["wd"])
+    torch.testing.assert_close(y.float(), dense.float(), **TOL[torch.float16])
+
+
+def test_config1_llama_fp32(oracle):
+    m = make_mlp(4096, 11008, 1, torch.float32, seed=0)
+    t = calibrate(m["wg"], [0.5])[0]
+    check_mlp_case(oracle, m, t, tag="llama-fp32-s0.5")
+
+
+def test_config3_mistral_bf16_heavy_tail(oracle):
+    m = make_mlp(4096, 14336, 1, torch.bfloat16, seed=3, heavy_tail=True)
+    for s, t in zip([0.5, 0.7], calibrate(m["wg"], [0.5, 0.7])):
+        check_mlp_case(oracle, m, t, tag=f"mistral-bf16-s{s}")
+
+
+@pytest.mark.parametrize("B", [2, 4, 8])
+def test_config4_small_batch_union(oracle, B):
+    m = make_mlp(4096, 11008, B, torch.float16, seed=4, corr=0.5)
+    t = calibrate(m["wg"], [0.5])[0]
+    r = check_mlp_case(oracle, m, t, tag=f"llama-fp16-B{B}")
+    union_sparsity = 1.0 - float(r["flag"].any(dim=0).float().mean())
+    row_sparsity = 1.0 - float(r["flag"].float().mean())
+    print(f"        B={B} per-row sparsity {row_sparsity:.3f} union sparsity {union_sparsity:.3f}", flush=True)
+    assert union_sparsity <= row_sparsity + 1e-6
+
+
+def test_reference_recipe_shapes(oracle):
+    """The reference's own test recipe: U(-0.5, 0.5) data, (4096 -> 14336), t = 0.2 / 0.3, B = 1 and 2
+    (flash_gemv/test/test_fuse_gemv_cmp.py:173-187, 442-524).  Only the gate / mask part is checked at t = 0.2;
+    the full pipeline at t = 0.3 in all three dtypes."""
+    m = make_mlp(4096, 14336, 1, torch.float16, seed=0, dist="uniform")
+    d = dev(m)
+    a, flag = capi.gate_flag(d["x"], d["wg"], 0.2)
+    assert torch.equal(flag, torch.abs(a) > 0.2)
+    for dtype in (torch.float16, torch.float32, torch.bfloat16):
+        m = make_mlp(4096, 14336, 2, dtype, seed=0, dist="uniform")
+        check_mlp_case(oracle, m, 0.3, tag=f"ref-recipe-{dtype}")
+
+
+def test_error_codes_on_device():
+    x = torch.zeros(1, 64, dtype=torch.float16, device="cuda")
+    w = torch.zeros(96, 64, dtype=torch.float16, device="cuda")
+    ws = _ws(1, 64, 96)
+    L = capi.lib()
+    p = capi._p
+    s = capi._stream(x)
+    small = torch.empty(256, dtype=torch.uint8, device="cuda")
+    y = torch.empty(1, 64, dtype=torch.float16, device="cuda")
+    assert L.cats_mlp(p(x), p(w), p(w), p(w), p(y), None, None, None, 1, 64, 96, 0, 0.1, p(small), 256, s) == 6  # workspace
+    assert L.cats_mlp(p(x), p(w), p(w), p(w), p(y), None, None, None, 9, 64, 96, 0, 0.1, p(ws.buf), ws.nbytes, s) == 4  # batch
+    assert L.cats_mlp(p(x), p(w), p(w), p(w), p(y), None, None, None, 1, 60, 96, 0, 0.1, p(ws.buf), ws.nbytes, s) == 3  # align
+    assert L.cats_mlp(p(x), p(w), p(w), p(w), p(y), None, None, None, 1, 64, 96, 7, 0.1, p(ws.buf), ws.nbytes, s) == 1  # dtype
+    assert L.cats_mlp(p(x), None, p(w), p(w), p(y), None, None, None, 1, 64, 96, 0, 0.1, p(ws.buf), ws.nbytes, s) == 5  # null
+    torch.cuda.synchronize()
