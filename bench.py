@@ -1,0 +1,283 @@
+#!/usr/bin/env python3
+"""Benchmark of the CATS sparse-MLP decode path on one MI355X.
+
+A "step" is one CATS MLP call (gate GEMV + SiLU + threshold + sparse up, then sparse down) on a
+Llama-2-7B-shaped layer (4096 -> 11008), fp16, batch 1, threshold at the 50th percentile of |SiLU(gate)| --
+the configuration the headline metric is quoted on.  Inputs are resident in HBM before the timed region.
+Steps rotate over several independent weight sets whose total size exceeds the 256 MB memory-side cache,
+so every step streams its weights from HBM.
+
+Prints ONE JSON line: per-layer latency (value, us), achieved HBM bandwidth on touched bytes, the same for
+sparsities 0/30/50/70/90 %, the dense fp16 GEMV MLP (stock PyTorch-ROCm F.linear) on the same GPU, a
+`roofline` object for the dominant kernel and a `cpu_baseline` object (the dense-masked PyTorch CATS MLP on
+this box's host cores).  `--decode` adds the 32-layer decode loop (tokens/s, CATS vs dense).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+H, I = 4096, 11008
+SPARSITIES = [0.0, 0.3, 0.5, 0.7, 0.9]
+
+
+def touched_bytes(sz, B, k):
+    """Algorithmic bytes of one CATS MLP call: all of W_gate, k rows each of W_up and W_down^T, x, y, a, the int32
+    index list and the count."""
+    return sz * H * I + 2 * sz * H * k + sz * B * (2 * H + I) + 4 * k + 4
+
+
+def stage_bytes(sz, B, k):
+    """Algorithmic bytes per launch of the two kernels: (gate+up, down)."""
+    gate_up = sz * H * I + sz * H * k + sz * B * H + I // 8 + 4 * B * k
+    down = sz * H * k + 4 * B * k + I // 8 + sz * B * H
+    return gate_up, down
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--sets", type=int, default=8, help="independent weight sets rotated through (cache defeat)")
+    ap.add_argument("--sparsity", type=float, default=0.5)
+    ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="time plain stream launches only")
+    ap.add_argument("--decode", action="store_true", help="also run the 32-layer decode loop (config 5)")
+    ap.add_argument("--down-groups", type=int, default=0)
+    ap.add_argument("--down-block", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the path needs no collective); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import torch.nn.functional as F
+
+    from cats_amd import capi
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    L = capi.lib()  # raises if the HIP library is missing: no fallback
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    dtype, sz, B = torch.float16, 2, 1
+    capi.set_tuning(0, args.down_groups, args.down_block, 0)
+
+    # ---- synthetic layer sets --------------------------------------------------------------------------------
+    g = torch.Generator(device="cuda").manual_seed(0)
+    sets = []
+    for _ in range(args.sets):
+        wg = (torch.randn(I, H, generator=g, device=dev) * 0.02).to(dtype)
+        wu = (torch.randn(I, H, generator=g, device=dev) * 0.02).to(dtype)
+        wd = (torch.randn(H, I, generator=g, device=dev) * 0.02).to(dtype)
+        sets.append(dict(wg=wg, wu=wu, wd=wd, wdt=wd.t().contiguous()))
+    x = torch.randn(B, H, generator=g, device=dev).to(dtype)
+    # thresholds: exact percentiles of |SiLU(X wg^T)| over 256 seeded calibration vectors (first set; the sets
+    # are identically distributed)
+    X = torch.randn(256, H, generator=g, device=dev)
+    act = F.silu(X @ sets[0]["wg"].float().t()).abs().flatten()
+    thr = {}
+    for s in SPARSITIES + [args.sparsity]:
+        thr[s] = -1.0 if s <= 0 else float(torch.kthvalue(act.cpu(), max(1, int(round(s * act.numel())))).values)
+    del X, act
+
+    ws = capi.Workspace(B, H, I)
+    y = torch.empty(B, H, dtype=dtype, device=dev)
+    count = torch.zeros(1, dtype=torch.int32, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def mlp_args(st, t, cnt=None):
+        return (p(x), p(st["wg"]), p(st["wu"]), p(st["wdt"]), p(y), None, None, cnt, B, H, I, capi.F16, ctypes.c_float(t),
+                p(ws.buf), ws.nbytes, stream)
+
+    def active_count(t):
+        ks = []
+        for st in sets:
+            capi.check(L.cats_mlp(*mlp_args(st, t, p(count))), "cats_mlp")
+            ks.append(int(count.item()))
+        return sum(ks) / len(ks)
+
+    def time_region(fn_step, steps, warmup):
+        """EXACTLY `steps` calls between two events on the launch stream, synchronised on both sides."""
+        for i in range(warmup):
+            fn_step(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            fn_step(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / steps  # us per step
+
+    def time_cats(t, steps, warmup, stages=0):
+        capi.set_tuning(0, args.down_groups, args.down_block, stages)
+        prepared = [mlp_args(st, t) for st in sets]
+        n = len(prepared)
+        fn = L.cats_mlp
+        us = time_region(lambda i: fn(*prepared[i % n]), steps, warmup)
+        capi.set_tuning(0, args.down_groups, args.down_block, 0)
+        return us
+
+    def time_cats_graph(t, steps, warmup):
+        """The same steps replayed from a HIP graph holding one step per weight set."""
+        prepared = [mlp_args(st, t) for st in sets]
+        n = len(prepared)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            sargs = [a[:-1] + (ctypes.c_void_p(side.cuda_stream),) for a in prepared]
+            for a in sargs:
+                L.cats_mlp(*a)
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                cap = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                for a in prepared:
+                    capi.check(L.cats_mlp(*(a[:-1] + (cap,))), "cats_mlp (capture)")
+        torch.cuda.synchronize()
+        reps, wreps = max(1, steps // n), max(1, warmup // n)
+        us = time_region(lambda i: graph.replay(), reps, wreps) / n
+        return us, reps * n
+
+    def time_dense(steps, warmup):
+        n = len(sets)
+
+        def step(i):
+            st = sets[i % n]
+            return F.linear(F.silu(F.linear(x, st["wg"])) * F.linear(x, st["wu"]), st["wd"])
+
+        return time_region(step, steps, warmup)
+
+    # ---- headline: 50 % sparsity ---------------------------------------------------------------------------------
+    t50 = thr[args.sparsity]
+    k50 = active_count(t50)
+    us_eager = time_cats(t50, args.steps, args.warmup)
+    if args.no_graph:
+        us_graph, graph_steps = None, 0
+    else:
+        us_graph, graph_steps = time_cats_graph(t50, args.steps, args.warmup)
+    us_gate_up = time_cats(t50, args.steps, args.warmup, stages=1)
+    us_down = time_cats(t50, args.steps, args.warmup, stages=2)
+    us_dense = time_dense(args.steps, args.warmup)
+    us = us_eager if us_graph is None else min(us_eager, us_graph)
+    launch = "stream" if (us_graph is None or us_eager <= us_graph) else "hipgraph"
+    steps_timed = args.steps if launch == "stream" else graph_steps
+    tb = touched_bytes(sz, B, k50)
+    b_gu, b_dn = stage_bytes(sz, B, k50)
+
+    sweep = []
+    if not args.no_sweep:
+        ssteps, swarm = max(200, args.steps // 4), max(50, args.warmup // 4)
+        for s in SPARSITIES:
+            k = active_count(thr[s])
+            u = time_cats(thr[s], ssteps, swarm)
+            if not args.no_graph:
+                u = min(u, time_cats_graph(thr[s], ssteps, swarm)[0])
+            b = touched_bytes(sz, B, k)
+            sweep.append(dict(target_sparsity=s, sparsity=round(1 - k / I, 4), us=round(u, 2), touched_MB=round(b / 1e6, 1),
+                              GBps=round(b / u * 1e-3, 1), hbm_frac=round(b / u * 1e-3 / HBM_PEAK_GBPS, 4),
+                              speedup_vs_dense=round(us_dense / u, 3)))
+
+    out = {
+        "metric": "CATS-MLP us/layer + achieved HBM GB/s (touched bytes); batch-1 decode tok/s",
+        "value": round(us, 3),
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": steps_timed,
+        "warmup": args.warmup,
+        "ms_per_step": round(us / 1e3, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "Llama-2-7B-shaped CATS MLP 4096->11008, fp16, batch 1, threshold at the 50th percentile of |SiLU(gate)|",
+                   "hidden": H, "intermediate": I, "batch": B, "target_sparsity": args.sparsity,
+                   "achieved_sparsity": round(1 - k50 / I, 4), "active_neurons": round(k50, 1), "weight_sets": args.sets,
+                   "launch": launch},
+        "touched_bytes": int(tb),
+        "achieved_GBps_touched": round(tb / us * 1e-3, 1),
+        "hbm_frac_touched": round(tb / us * 1e-3 / HBM_PEAK_GBPS, 4),
+        "us_stream_launch": round(us_eager, 3),
+        "us_hipgraph": None if us_graph is None else round(us_graph, 3),
+        "dense_fp16_us": round(us_dense, 3),
+        "dense_GBps": round(3 * sz * H * I / us_dense * 1e-3, 1),
+        "speedup_vs_dense": round(us_dense / us, 3),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "cats::rows_kernel<F16,B=1,kGateUp> (gate GEMV + SiLU + threshold + sparse up)",
+            "achieved": round(b_gu / us_gate_up * 1e-3, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(b_gu / us_gate_up * 1e-3 / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "bytes_per_launch": int(b_gu),
+            "us_per_launch": round(us_gate_up, 3),
+            "second_kernel": {"kernel": "cats::down_kernel<F16,B=1> (sparse neuron-major down)", "bytes_per_launch": int(b_dn),
+                              "us_per_launch": round(us_down, 3), "achieved": round(b_dn / us_down * 1e-3, 1),
+                              "frac": round(b_dn / us_down * 1e-3 / HBM_PEAK_GBPS, 4)},
+            "note": "per-kernel times are back-to-back launches of that kernel alone (launch gap included); value is the whole call",
+        },
+        "sweep": sweep,
+    }
+
+    if args.decode:
+        from cats_amd import decoder
+
+        out["decode"] = decoder.bench_decode(prompt_len=128, gen_len=256, sparsity=0.5)
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(torch, F, thr[0.5] if 0.5 in thr else t50)
+
+    print(json.dumps(out))
+
+
+def cpu_baseline(torch, F, t):
+    """The dense-masked PyTorch CATS MLP (the reference's sp_method 0 branch) in fp32 on the host cores."""
+    from oracle import cats_oracle
+
+    ncores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    threads = min(ncores, int(os.environ.get("OMP_NUM_THREADS", ncores)))
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(0)
+    wg = torch.randn(I, H, generator=g) * 0.02
+    wu = torch.randn(I, H, generator=g) * 0.02
+    wd = torch.randn(H, I, generator=g) * 0.02
+    x = torch.randn(1, 1, H, generator=g)
+    for _ in range(3):
+        cats_oracle.torch_cats_mlp(x, wg, wu, wd, t)
+    times = []
+    t_end = time.perf_counter() + 12.0
+    while len(times) < 20 or (time.perf_counter() < t_end and len(times) < 400):
+        t0 = time.perf_counter()
+        cats_oracle.torch_cats_mlp(x, wg, wu, wd, t)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    cpu = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                cpu = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {"value": round(med * 1e6, 1), "unit": "us/layer", "cores": threads, "kind": "port",
+            "sample": f"{len(times)} calls of the fp32 dense-masked PyTorch CATS MLP (4096->11008, batch 1), median; cpu: {cpu}",
+            "GBps_dense_bytes": round(3 * 4 * H * I / med * 1e-9, 1)}
+
+
+if __name__ == "__main__":
+    main()

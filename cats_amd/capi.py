@@ -49,7 +49,7 @@ def lib() -> ctypes.CDLL:
         L.cats_gate_up.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp]; L.cats_gate_up.restype = i32
         L.cats_mlp.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_mlp.restype = i32
         L.cats_mlp_rowmajor_down.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_mlp_rowmajor_down.restype = i32
-        L.cats_set_tuning.argtypes = [i32, i32, i32]; L.cats_set_tuning.restype = i32
+        L.cats_set_tuning.argtypes = [i32, i32, i32, i32]; L.cats_set_tuning.restype = i32
         _lib = L
     return _lib
 
@@ -160,5 +160,5 @@ def mlp_rowmajor_down(x, wgate, wup, wdown, threshold, ws: Workspace):
     return y
 
 
-def set_tuning(gate_variant=0, down_groups=0, down_block=0):
-    lib().cats_set_tuning(int(gate_variant), int(down_groups), int(down_block))
+def set_tuning(gate_variant=0, down_groups=0, down_block=0, stages=0):
+    lib().cats_set_tuning(int(gate_variant), int(down_groups), int(down_block), int(stages))

@@ -19,7 +19,11 @@ template <> hipError_t launch_down<F32>(int, bool, const DownArgs&, int, hipStre
 
 namespace {
 
-Tuning g_tuning = {0, 0, 0};
+Tuning g_tuning = {0, 0, 0, 0};
+#ifdef CATS_TIMING
+long long* g_tbuf_rows = nullptr;
+long long* g_tbuf_down = nullptr;
+#endif
 
 constexpr int kMaxSlabs = 128;
 constexpr size_t kCounterBytes = 1024;  // done[128] | arrive | pad
@@ -47,18 +51,20 @@ __global__ void pack_flags_kernel(const uint8_t* flag, int nb, int I, uint8_t* m
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct WsLayout {
-  size_t counters, mask, z32, zt, y32, atmp, total;
+  size_t counters, mask, z32, zt, partial, atmp, total;
 };
 
+constexpr int kMaxGroups = 64;  // neuron groups of the sparse down kernel; bounds the partial-sum scratch
+
 // The carving depends on (H, I) only -- every region is sized for CATS_MAX_BATCH rows -- so calls with
-// different batch sizes can share one workspace and the regions that must stay zero (counters, y32) never
-// move onto bytes another call has dirtied.
+// different batch sizes can share one workspace and the region that must stay zero (the counters) never
+// moves onto bytes another call has dirtied.
 WsLayout ws_layout(int H, int I) {
   WsLayout l;
   const int B = CATS_MAX_BATCH;
   size_t o = 0;
   l.counters = o; o += kCounterBytes;
-  l.y32 = o;      o += align_up((size_t)B * H * 4, 256);
+  l.partial = o;  o += align_up((size_t)kMaxGroups * B * ((size_t)(H + 511) / 512 * 512) * 4, 256);
   l.mask = o;     o += align_up((size_t)((I + 63) / 64) * 8, 256);
   l.z32 = o;      o += align_up((size_t)B * I * 4, 256);
   l.zt = o;       o += align_up((size_t)B * I * 4, 256);
@@ -154,7 +160,11 @@ void fill_rows(RowsArgs& a, const void* x, const void* w, int K, int N, int nb, 
   a.nch = (a.row_vecs + kWave - 1) / kWave;
 }
 
-int do_rows(int mode, int dtype, const RowsArgs& a, hipStream_t s) {
+int do_rows(int mode, int dtype, const RowsArgs& a_in, hipStream_t s) {
+  RowsArgs a = a_in;
+#ifdef CATS_TIMING
+  a.tbuf = g_tbuf_rows;
+#endif
   const int bt = batch_template(a.nb);
   hipError_t e;
   if (dtype == CATS_F16) e = launch_rows<F16>(mode, bt, a, s);
@@ -170,26 +180,31 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   memset(&d, 0, sizeof(d));
   d.wd = (const u32x4*)wdown_t;
   d.z = z;
-  d.mask = (const uint64_t*)(ws + l.mask);
+  d.mask = (const uint8_t*)(ws + l.mask);
   d.y32 = y32;
   d.y_out = y_out;
+  d.partial = (float*)(ws + l.partial);
   d.done = (uint32_t*)(ws + l.counters);
   d.count_out = count_out;
   d.H = H; d.I = I; d.nb = B;
   d.row_vecs = H / vec_elems(dtype);
   d.nslab = (d.row_vecs + kWave - 1) / kWave;
-  d.nwords = (I + 63) / 64;
-  if (d.nslab > kMaxSlabs || I > CATS_MAX_INTERMEDIATE) return CATS_ERR_SHAPE;
-  int ngroup = g_tuning.down_groups > 0 ? g_tuning.down_groups : 256 / d.nslab;
-  if (ngroup < 1) ngroup = 1;
-  if (ngroup > I) ngroup = I;
-  d.ngroup = ngroup;
-  d.ncap = (I + ngroup - 1) / ngroup + 1;
+  if (d.nslab > kMaxSlabs) return CATS_ERR_SHAPE;
   int block = g_tuning.down_block > 0 ? g_tuning.down_block : 1024;
-  if (block < 64) block = 64;
+  if (block < 128) block = 128;  // wave 0 builds the index list, the others stage z
   if (block > 1024) block = 1024;
   block = block / 64 * 64;
   const int bt = batch_template(B);
+  // about one workgroup per CU over all slabs; more groups if a group's list and z would not fit in LDS
+  int ngroup = g_tuning.down_groups > 0 ? g_tuning.down_groups : 256 / d.nslab;
+  if (ngroup < 1) ngroup = 1;
+  if (ngroup > kMaxGroups) ngroup = kMaxGroups;
+  d.chunk = ((I + ngroup - 1) / ngroup + 7) / 8 * 8;
+  if ((size_t)d.chunk * (1 + bt) * 4 > 96 * 1024) return CATS_ERR_SHAPE;  // a group's list and z must fit in LDS
+  d.ngroup = (I + d.chunk - 1) / d.chunk;
+#ifdef CATS_TIMING
+  d.tbuf = g_tbuf_down;
+#endif
   hipError_t e;
   if (dtype == CATS_F16) e = launch_down<F16>(bt, zf32, d, block, s);
   else if (dtype == CATS_BF16) e = launch_down<BF16>(bt, zf32, d, block, s);
@@ -210,13 +225,17 @@ using namespace cats;
 
 extern "C" {
 
+#ifdef CATS_TIMING
+void cats_timing_buffers(void* rows, void* down) { g_tbuf_rows = (long long*)rows; g_tbuf_down = (long long*)down; }
+#endif
+
 int cats_version(void) { return 100; }
 
 const char* cats_status_string(int status) {
   switch (status) {
     case CATS_OK: return "ok";
     case CATS_ERR_DTYPE: return "unsupported dtype (expected 0=fp16, 1=bf16, 2=fp32)";
-    case CATS_ERR_SHAPE: return "unsupported shape (H, I must be positive; I <= 65536; H <= 128 slabs of 64 x 16 bytes)";
+    case CATS_ERR_SHAPE: return "unsupported shape (H, I must be positive; H <= 128 slabs of 64 x 16 bytes)";
     case CATS_ERR_ALIGN: return "pointer or row pitch not 16-byte aligned";
     case CATS_ERR_BATCH: return "unsupported batch (1..8 rows)";
     case CATS_ERR_NULL: return "required pointer is NULL";
@@ -226,10 +245,11 @@ const char* cats_status_string(int status) {
   return "unknown status";
 }
 
-int cats_set_tuning(int gate_variant, int down_groups, int down_block) {
+int cats_set_tuning(int gate_variant, int down_groups, int down_block, int stages) {
   g_tuning.gate_variant = gate_variant;
   g_tuning.down_groups = down_groups;
   g_tuning.down_block = down_block;
+  g_tuning.stages = stages;
   return CATS_OK;
 }
 
@@ -319,7 +339,7 @@ int cats_down_flag(const void* z, const void* wdown_t, const uint8_t* flag, floa
   hipLaunchKernelGGL(pack_flags_kernel, dim3((nbytes + 255) / 256), dim3(256), 0, (hipStream_t)stream, flag, B, I,
                      (uint8_t*)ws + l.mask, nbytes);
   if (hipGetLastError() != hipSuccess) return CATS_ERR_LAUNCH;
-  float* acc = y_f32 ? y_f32 : (float*)((char*)ws + l.y32);
+  float* acc = y_f32;
   return do_down(z, false, wdown_t, acc, y_out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
 }
 
@@ -355,9 +375,12 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
   a.mask_out = (uint8_t*)ws + l.mask;
   a.flag_out = flag_out;
   a.t = round_through(dtype, threshold);
-  st = do_rows(kGateUp, dtype, a, (hipStream_t)stream);
-  if (st) return st;
-  float* acc = y_f32 ? y_f32 : (float*)((char*)ws + l.y32);
+  if (g_tuning.stages != 2) {
+    st = do_rows(kGateUp, dtype, a, (hipStream_t)stream);
+    if (st) return st;
+  }
+  if (g_tuning.stages == 1) return CATS_OK;
+  float* acc = y_f32;
   return do_down(a.z32_out, true, wdown_t, acc, y_out, count_out, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
 }
 

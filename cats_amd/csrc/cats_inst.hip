@@ -60,7 +60,7 @@ template <class DT, int B, bool ZF32>
 hipError_t launch_down_one(const DownArgs& a, int block, hipStream_t stream) {
   auto kern = down_kernel<DT, B, ZF32, kDownU>;
   const int nwaves = block / kWave;
-  const size_t lds = ((size_t)a.ncap * (1 + B) + (size_t)nwaves * kWave * DT::VEC) * sizeof(float);
+  const size_t lds = ((size_t)a.chunk * (1 + B) + (size_t)nwaves * kWave * DT::VEC) * sizeof(float);
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;

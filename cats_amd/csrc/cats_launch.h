@@ -11,6 +11,7 @@ struct Tuning {
   int gate_variant;  // reserved for alternative gate kernels; 0 = default
   int down_groups;   // 0 = default (about one workgroup per CU over all slabs)
   int down_block;    // 0 = default (1024 threads)
+  int stages;        // cats_mlp only: 0 = both launches, 1 = gate+up only, 2 = down only (profiling)
 };
 
 // Returns hipSuccess or the launch error.  `mode` is a RowsMode; bt (1, 2, 4 or 8) the compile-time batch.

@@ -38,36 +38,52 @@ struct RowsArgs {
   int nch;               // 64-lane vector chunks per row: ceil(K / (64 * VEC))
   int row_vecs;          // K / VEC
   float t;               // threshold, already rounded through dtype
+#ifdef CATS_TIMING
+  long long* tbuf;       // [gridDim][8] wall-clock stamps (100 MHz) at phase boundaries, development builds only
+#endif
 };
 
-// Dot products of R weight rows against the nb staged x rows.  acc[r][b] ends up wave-uniform.
+#ifdef CATS_TIMING
+#define CATS_RSTAMP(slot) do { if (p.tbuf && threadIdx.x == 0) p.tbuf[(size_t)blockIdx.x * 8 + (slot)] = wall_clock64(); } while (0)
+#else
+#define CATS_RSTAMP(slot) do { } while (0)
+#endif
+
+// One block of weight loads: CB chunks of 64 lanes x 16 bytes for each of the R rows, issued back to back so
+// they are all in flight together.  Loads are never predicated per lane: lanes past the end of a row re-read
+// its last vector and later meet a zero in x (the LDS copy of x is zero-padded to whole blocks of CB chunks).
+template <int R, int CB, bool FULL>
+__device__ __forceinline__ void rows_issue(const u32x4* __restrict__ w, const int (&row)[R], const bool (&on)[R], int c0,
+                                           const RowsArgs& p, int lane, u32x4 (&wv)[R][CB]) {
+  const int vlast = p.row_vecs - 1;
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    if (on[r]) {  // wave-uniform
+      const u32x4* wr = w + (size_t)row[r] * p.row_vecs;
+#pragma unroll
+      for (int cc = 0; cc < CB; cc++) {
+        const int v = (c0 + cc) * kWave + lane;
+        wv[r][cc] = load_stream(wr + (FULL ? v : min(v, vlast)));
+      }
+    }
+  }
+}
+
+// Dot products of R weight rows against the nb staged x rows.  acc[r][b] ends up wave-uniform.  `wv` holds the
+// loads of the first block if `preissued` (the caller started them before x was staged), else it is scratch.
 template <class DT, int B, int R, int CB, bool FULL, bool XLDS>
 __device__ __forceinline__ void rows_dot(const u32x4* __restrict__ w, const int (&row)[R], const bool (&on)[R],
                                          const u32x4* xs, const u32x4* __restrict__ xg, const RowsArgs& p, int lane,
-                                         float (&acc)[R][B]) {
+                                         u32x4 (&wv)[R][CB], bool preissued, float (&acc)[R][B]) {
 #pragma unroll
   for (int r = 0; r < R; r++)
 #pragma unroll
     for (int b = 0; b < B; b++) acc[r][b] = 0.f;
 
-  // Loads are never predicated per lane: lanes past the end of a row re-read its last vector and meet a
-  // zero in x (the LDS copy of x is zero-padded to whole blocks of CB chunks), so a block of CB loads per
-  // row is issued back to back and stays in flight together.
   const int vlast = p.row_vecs - 1;
   const int nchp = (p.nch + CB - 1) / CB * CB;
   for (int c0 = 0; c0 < p.nch; c0 += CB) {
-    u32x4 wv[R][CB];
-#pragma unroll
-    for (int r = 0; r < R; r++) {
-      if (on[r]) {  // wave-uniform
-        const u32x4* wr = w + (size_t)row[r] * p.row_vecs;
-#pragma unroll
-        for (int cc = 0; cc < CB; cc++) {
-          const int v = (c0 + cc) * kWave + lane;
-          wv[r][cc] = load_stream(wr + (FULL ? v : min(v, vlast)));
-        }
-      }
-    }
+    if (!(preissued && c0 == 0)) rows_issue<R, CB, FULL>(w, row, on, c0, p, lane, wv);
 #pragma unroll
     for (int cc = 0; cc < CB; cc++) {
       const int v = (c0 + cc) * kWave + lane;
@@ -108,18 +124,7 @@ __global__ __launch_bounds__(WAVES* kWave) void rows_kernel(RowsArgs p) {
   constexpr int kRowsPerBlock = WAVES * R;
   static_assert(kRowsPerBlock % 8 == 0 && kRowsPerBlock <= 32, "mask bytes are assembled in one 32-bit LDS word");
 
-  if (XLDS) {
-    const int nchv = (p.nch + CB - 1) / CB * CB * kWave;  // padded vectors per x row
-    for (int i = threadIdx.x; i < B * nchv; i += kThreads) {
-      const int b = i / nchv, v = i - b * nchv;
-      u32x4 val = zero4();
-      if (b < p.nb && v < p.row_vecs) val = p.x[(size_t)b * p.row_vecs + v];
-      xs[i] = val;
-    }
-  }
-  if (threadIdx.x == 0) s_maskbits = 0u;
-  __syncthreads();
-
+  CATS_RSTAMP(0);
   const int row0 = (blockIdx.x * WAVES + wave) * R;
   int row[R];
   bool on[R];
@@ -128,6 +133,40 @@ __global__ __launch_bounds__(WAVES* kWave) void rows_kernel(RowsArgs p) {
     row[r] = row0 + r < p.N ? row0 + r : p.N - 1;
     on[r] = row0 + r < p.N;
   }
+
+  // Staging order matters: memory returns are counted in issue order, so the x loads go out first, then the
+  // first block of weight loads, and only the x values are waited for before the LDS writes and the barrier --
+  // the weight loads stay in flight across both.
+  u32x4 wv[R][CB];
+  constexpr int kXPre = 2;  // x vectors per thread fetched ahead of the weights (covers B*H*sizeof <= 8 KiB per 256 threads)
+  const int nchv = (p.nch + CB - 1) / CB * CB * kWave;  // padded vectors per x row
+  u32x4 xpre[kXPre];
+  if (XLDS) {
+#pragma unroll
+    for (int k = 0; k < kXPre; k++) {
+      const int i = threadIdx.x + k * kThreads;
+      const int b = B == 1 ? 0 : i / nchv, v = i - b * nchv;
+      xpre[k] = zero4();
+      if (i < B * nchv && b < p.nb && v < p.row_vecs) xpre[k] = p.x[(size_t)b * p.row_vecs + v];
+    }
+  }
+  if (MODE != kUp) rows_issue<R, CB, FULL>(p.w, row, on, 0, p, lane, wv);
+  if (XLDS) {
+#pragma unroll
+    for (int k = 0; k < kXPre; k++) {
+      const int i = threadIdx.x + k * kThreads;
+      if (i < B * nchv) xs[i] = xpre[k];
+    }
+    for (int i = threadIdx.x + kXPre * kThreads; i < B * nchv; i += kThreads) {
+      const int b = i / nchv, v = i - b * nchv;
+      u32x4 val = zero4();
+      if (b < p.nb && v < p.row_vecs) val = p.x[(size_t)b * p.row_vecs + v];
+      xs[i] = val;
+    }
+  }
+  if (threadIdx.x == 0) s_maskbits = 0u;
+  __syncthreads();
+  CATS_RSTAMP(1);
 
   float a[R][B];       // gate activation, rounded through dtype
   bool act[R][B];      // per batch row flag
@@ -149,7 +188,7 @@ __global__ __launch_bounds__(WAVES* kWave) void rows_kernel(RowsArgs p) {
     }
   } else {
     float g[R][B];
-    rows_dot<DT, B, R, CB, FULL, XLDS>(p.w, row, on, xs, p.x, p, lane, g);
+    rows_dot<DT, B, R, CB, FULL, XLDS>(p.w, row, on, xs, p.x, p, lane, wv, true, g);
     if (MODE == kGemv) {
       if (lane == 0) {
         st* out = (st*)p.zt_out;
@@ -194,9 +233,10 @@ __global__ __launch_bounds__(WAVES* kWave) void rows_kernel(RowsArgs p) {
     }
   }
 
+  CATS_RSTAMP(2);
   if (MODE == kGateUp || MODE == kUp) {
     float u[R][B];
-    rows_dot<DT, B, R, CB, FULL, XLDS>(MODE == kGateUp ? p.w2 : p.w, row, any, xs, p.x, p, lane, u);
+    rows_dot<DT, B, R, CB, FULL, XLDS>(MODE == kGateUp ? p.w2 : p.w, row, any, xs, p.x, p, lane, wv, false, u);
     if (lane == 0) {
 #pragma unroll
       for (int r = 0; r < R; r++)
@@ -213,6 +253,7 @@ __global__ __launch_bounds__(WAVES* kWave) void rows_kernel(RowsArgs p) {
     }
   }
 
+  CATS_RSTAMP(3);
   if (MODE == kGate || MODE == kGateUp) {
     if (p.mask_out) {
       __syncthreads();

@@ -323,8 +323,8 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> cats_mlp_stats_op(const at::Tenso
   return {out, flags, count};
 }
 
-void cats_set_tuning_op(int64_t gate_variant, int64_t down_groups, int64_t down_block) {
-  cats_set_tuning((int)gate_variant, (int)down_groups, (int)down_block);
+void cats_set_tuning_op(int64_t gate_variant, int64_t down_groups, int64_t down_block, int64_t stages) {
+  cats_set_tuning((int)gate_variant, (int)down_groups, (int)down_block, (int)stages);
 }
 
 }  // namespace

@@ -54,7 +54,6 @@ typedef enum {
 } cats_status_t;
 
 #define CATS_MAX_BATCH 8
-#define CATS_MAX_INTERMEDIATE 65536 /* sparse down kernel scans I/64 mask words in one block */
 
 /* Library identification / error text.  No reference counterpart (the reference printf()s and exit()s:
  * flash_gemv/csrc/cuda/fuse_gemv_cmp_cuda.cu:25-33,2397-2400). */
@@ -130,8 +129,10 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
 int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out,
                            int B, int H, int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream);
 
-/* Launch-shape knobs for experiments and profiling; 0 keeps the built-in choice.  Not in the reference. */
-int cats_set_tuning(int gate_variant, int down_groups, int down_block);
+/* Launch-shape knobs for experiments and profiling; 0 keeps the built-in choice.  `stages` restricts cats_mlp
+ * to one of its two launches (1 = gate+up only, 2 = sparse down only, over whatever mask and z the workspace
+ * holds from the previous full call) so each kernel can be timed alone.  Process-global; not in the reference. */
+int cats_set_tuning(int gate_variant, int down_groups, int down_block, int stages);
 
 #ifdef __cplusplus
 }
