@@ -1,0 +1,292 @@
+"""A Llama-2-7B-architecture decoder around the CATS MLP, for the end-to-end decode measurement.
+
+The reference never defines the decoder itself: it subclasses the HF Llama / Mistral models and only swaps
+``layer.mlp`` (experiments/models/sparse_silu/ugly_utils.py:119-131).  What is restated here are the conventions
+its tree spells out: decoder layer order ``h += attn(input_layernorm(h)); h += mlp(post_attention_layernorm(h))``
+(ugly_utils.py:1016-1057), rotate-half RoPE and eager attention with an fp32 softmax
+(experiments/models/sparse_mistral/sparse_silu.py:280-312, 756-832), and the timing rule of the patched
+``generate()``: tokens 2..N only, tok/s = (N - 1) / elapsed (experiments/time_util_nofile.py:2902-2904, 2984-2994).
+Everything except the MLP uses stock PyTorch-ROCm ops, so dense-vs-CATS differences isolate the MLP path.
+The decode step is shape-static (fixed-size KV cache, position kept on the device) so it can be replayed from a
+HIP graph.
+"""
+from __future__ import annotations
+
+import math
+import time
+from dataclasses import dataclass
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .mlp import CatsMLP
+
+
+@dataclass
+class DecoderConfig:
+    hidden_size: int = 4096
+    intermediate_size: int = 11008
+    num_layers: int = 32
+    num_heads: int = 32
+    vocab_size: int = 32000
+    rms_eps: float = 1e-5
+    rope_theta: float = 10000.0
+    max_len: int = 512
+
+    @property
+    def head_dim(self):
+        return self.hidden_size // self.num_heads
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim, eps, dtype, device):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim, dtype=dtype, device=device))
+        self.eps = eps
+
+    def forward(self, x):
+        v = x.float()
+        v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + self.eps)
+        return self.weight * v.to(x.dtype)
+
+
+def rotate_half(x):
+    d = x.shape[-1] // 2
+    return torch.cat((-x[..., d:], x[..., :d]), dim=-1)
+
+
+class Attention(nn.Module):
+    def __init__(self, cfg: DecoderConfig, dtype, device):
+        super().__init__()
+        Hd = cfg.hidden_size
+        kw = dict(bias=False, dtype=dtype, device=device)
+        self.cfg = cfg
+        self.q_proj, self.k_proj, self.v_proj, self.o_proj = (nn.Linear(Hd, Hd, **kw) for _ in range(4))
+        self.k_cache = None
+        self.v_cache = None
+
+    def reset_cache(self, batch, dtype, device):
+        c = self.cfg
+        self.k_cache = torch.zeros(batch, c.num_heads, c.max_len, c.head_dim, dtype=dtype, device=device)
+        self.v_cache = torch.zeros_like(self.k_cache)
+
+    def forward(self, h, cos, sin, positions, mask):
+        """h (B, q, H); cos/sin (q, head_dim); positions (q,) int64 cache slots; mask (q, max_len) additive."""
+        c = self.cfg
+        B, q, _ = h.shape
+        shp = (B, q, c.num_heads, c.head_dim)
+        qh = self.q_proj(h).view(shp).transpose(1, 2)
+        kh = self.k_proj(h).view(shp).transpose(1, 2)
+        vh = self.v_proj(h).view(shp).transpose(1, 2)
+        qh = qh * cos + rotate_half(qh) * sin
+        kh = kh * cos + rotate_half(kh) * sin
+        self.k_cache.index_copy_(2, positions, kh)
+        self.v_cache.index_copy_(2, positions, vh)
+        att = torch.matmul(qh, self.k_cache.transpose(2, 3)) / math.sqrt(c.head_dim) + mask
+        att = torch.softmax(att, dim=-1, dtype=torch.float32).to(h.dtype)
+        out = torch.matmul(att, self.v_cache).transpose(1, 2).reshape(B, q, c.hidden_size)
+        return self.o_proj(out)
+
+
+class DecoderLayer(nn.Module):
+    def __init__(self, cfg, dtype, device):
+        super().__init__()
+        self.input_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_eps, dtype, device)
+        self.self_attn = Attention(cfg, dtype, device)
+        self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_eps, dtype, device)
+        self.mlp = CatsMLP(cfg.hidden_size, cfg.intermediate_size, dtype=dtype, device=device)
+
+    def forward(self, h, cos, sin, positions, mask):
+        h = h + self.self_attn(self.input_layernorm(h), cos, sin, positions, mask)
+        return h + self.mlp(self.post_attention_layernorm(h))
+
+
+class LlamaDecoder(nn.Module):
+    """Random-init decoder-only transformer in the Llama-2 layout (no biases, untied lm_head)."""
+
+    def __init__(self, cfg: DecoderConfig, dtype=torch.float16, device="cuda", seed=0, init_std=0.02):
+        super().__init__()
+        self.cfg, self.dtype = cfg, dtype
+        self.embed_tokens = nn.Embedding(cfg.vocab_size, cfg.hidden_size, dtype=dtype, device=device)
+        self.layers = nn.ModuleList(DecoderLayer(cfg, dtype, device) for _ in range(cfg.num_layers))
+        self.norm = RMSNorm(cfg.hidden_size, cfg.rms_eps, dtype, device)
+        self.lm_head = nn.Linear(cfg.hidden_size, cfg.vocab_size, bias=False, dtype=dtype, device=device)
+        g = torch.Generator(device=device).manual_seed(seed)
+        with torch.no_grad():
+            for name, p in self.named_parameters():
+                if p.dim() == 2:
+                    p.copy_((torch.randn(p.shape, generator=g, device=device, dtype=torch.float32) * init_std).to(dtype))
+        inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, cfg.head_dim, 2, device=device).float() / cfg.head_dim))
+        ang = torch.outer(torch.arange(cfg.max_len, device=device).float(), inv)
+        emb = torch.cat((ang, ang), dim=-1)
+        self.register_buffer("cos_table", emb.cos().to(dtype), persistent=False)
+        self.register_buffer("sin_table", emb.sin().to(dtype), persistent=False)
+
+    def reset_cache(self, batch=1):
+        dev = self.embed_tokens.weight.device
+        for layer in self.layers:
+            layer.self_attn.reset_cache(batch, self.dtype, dev)
+
+    def forward(self, tokens, positions):
+        """tokens (B, q) int64; positions (q,) int64 -> logits (B, q, vocab).  Causal over cache slots <= position."""
+        cfg = self.cfg
+        h = self.embed_tokens(tokens)
+        cos, sin = self.cos_table[positions], self.sin_table[positions]
+        slots = torch.arange(cfg.max_len, device=tokens.device)
+        mask = torch.zeros(positions.numel(), cfg.max_len, dtype=self.dtype, device=tokens.device)
+        mask.masked_fill_(slots[None, :] > positions[:, None], float("-inf"))
+        for layer in self.layers:
+            h = layer(h, cos, sin, positions, mask)
+        return self.lm_head(self.norm(h))
+
+    # ---- MLP mode switches ----
+    def set_mlp_mode(self, mode: str):
+        """"dense": plain SwiGLU.  "cats_torch": dense-masked PyTorch.  "cats": the two-launch HIP path.
+        "cats_rowmajor": flag_gemv_gemv_inner* (HF-layout down).  "cats_split": torch gate + HIP sparse up / down."""
+        for layer in self.layers:
+            m = layer.mlp
+            if mode == "dense":
+                m.is_profile, m.kill_sparse_swish_outputs = False, False
+            elif mode == "cats_torch":
+                m.is_profile, m.sp_method = True, 0
+            elif mode in ("cats", "cats_split", "cats_rowmajor"):
+                m.prepare_decode({"cats": 3, "cats_split": 2, "cats_rowmajor": 1}[mode])
+            else:
+                raise ValueError(mode)
+
+    @torch.no_grad()
+    def calibrate(self, sparsity: float, n_seq: int = 64, seq_len: int = 128, seed: int = 1, chunk: int = 8):
+        """Per-layer thresholds at an exact percentile of |SiLU(gate)| over n_seq seeded random-token sequences, run
+        through the dense model (the reference collects its histograms before thresholds are set)."""
+        dev = self.embed_tokens.weight.device
+        g = torch.Generator(device=dev).manual_seed(seed)
+        acts = [[] for _ in self.layers]
+        hooks = []
+        for i, layer in enumerate(self.layers):
+            hooks.append(layer.mlp.gate_proj.register_forward_hook(
+                lambda mod, inp, out, i=i: acts[i].append(F.silu(out).abs().flatten().float()[::4].clone())))
+        self.set_mlp_mode("dense")
+        positions = torch.arange(seq_len, device=dev)
+        for s in range(0, n_seq, chunk):
+            toks = torch.randint(0, self.cfg.vocab_size, (min(chunk, n_seq - s), seq_len), generator=g, device=dev)
+            self.reset_cache(toks.shape[0])
+            self.forward(toks, positions)
+        for h in hooks:
+            h.remove()
+        thresholds = []
+        for i, layer in enumerate(self.layers):
+            a = torch.cat(acts[i])
+            k = max(1, int(round(sparsity * a.numel())))
+            t = float(torch.kthvalue(a, k).values) if sparsity > 0 else -1.0
+            layer.mlp.dead_threshold = t
+            thresholds.append(t)
+            acts[i] = None
+        return thresholds
+
+    @torch.no_grad()
+    def generate_greedy(self, prompt, gen_len: int, use_graph: bool = True):
+        """Greedy decode; returns (tokens (gen_len,), seconds for tokens 2..gen_len).  The first generated token
+        comes from the prefill and is not timed (experiments/time_util_nofile.py:2902-2904)."""
+        dev = prompt.device
+        P = prompt.shape[1]
+        assert P + gen_len <= self.cfg.max_len
+        self.reset_cache(1)
+        logits = self.forward(prompt, torch.arange(P, device=dev))
+        tok = logits[:, -1].argmax(-1, keepdim=True)                     # token 1
+        out = torch.zeros(gen_len, dtype=torch.int64, device=dev)
+        out[0] = tok[0, 0]
+        pos = torch.full((1,), P, dtype=torch.int64, device=dev)
+        step_idx = torch.ones(1, dtype=torch.int64, device=dev)
+
+        def step():
+            lg = self.forward(tok, pos)
+            nxt = lg[:, -1].argmax(-1, keepdim=True)
+            tok.copy_(nxt)
+            out.index_copy_(0, step_idx, nxt[0])
+            pos.add_(1)
+            step_idx.add_(1)
+
+        graph = None
+        if use_graph:
+            snap = [t.clone() for t in (tok, pos, step_idx, out)]
+            caches = [(l.self_attn.k_cache.clone(), l.self_attn.v_cache.clone()) for l in self.layers]
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()                                                   # warm-up on the capture stream (allocations)
+                side.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    step()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            for t, s in zip((tok, pos, step_idx, out), snap):            # rewind the two steps spent on capture
+                t.copy_(s)
+            for l, (k, v) in zip(self.layers, caches):
+                l.self_attn.k_cache.copy_(k)
+                l.self_attn.v_cache.copy_(v)
+            del caches
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(gen_len - 1):
+            if graph is not None:
+                graph.replay()
+            else:
+                step()
+        e1.record()
+        torch.cuda.synchronize()
+        return out.clone(), e0.elapsed_time(e1) * 1e-3
+
+
+def bench_decode(prompt_len=128, gen_len=256, sparsity=0.5, num_layers=32, seed=0, use_graph=True, cfg=None):
+    """Config 5: random-init fp16 Llama-2-7B architecture, batch 1, uniform-random prompt, greedy decode.
+    Returns tok/s for the dense MLP and the CATS MLP (HIP path) and their ratio."""
+    cfg = cfg or DecoderConfig(num_layers=num_layers, max_len=prompt_len + gen_len)
+    t0 = time.time()
+    model = LlamaDecoder(cfg, torch.float16, "cuda", seed=seed).eval()
+    thresholds = model.calibrate(sparsity)
+    g = torch.Generator(device="cuda").manual_seed(seed + 7)
+    prompt = torch.randint(0, cfg.vocab_size, (1, prompt_len), generator=g, device="cuda")
+    res = {"layers": cfg.num_layers, "prompt_len": prompt_len, "gen_len": gen_len, "target_sparsity": sparsity,
+           "launch": "hipgraph" if use_graph else "stream", "setup_s": None}
+    toks = {}
+    for mode in ("dense", "cats"):
+        model.set_mlp_mode(mode)
+        model.generate_greedy(prompt, min(gen_len, 8), use_graph=False)          # warm-up (workspaces, kernels)
+        out, secs = model.generate_greedy(prompt, gen_len, use_graph=use_graph)
+        toks[mode] = out
+        res[f"{mode}_tok_s"] = round((gen_len - 1) / secs, 2)
+        res[f"{mode}_ms_per_token"] = round(secs / (gen_len - 1) * 1e3, 4)
+    res["speedup"] = round(res["cats_tok_s"] / res["dense_tok_s"], 3)
+    # achieved union sparsity over the generated tokens is not observable without a sync per layer; report the
+    # calibration target and the mean threshold instead
+    res["mean_threshold"] = round(sum(thresholds) / len(thresholds), 5)
+    res["setup_s"] = round(time.time() - t0, 1)
+    return res
+
+
+@torch.no_grad()
+def cpu_decode_baseline(num_layers=4, gen_len=8, prompt_len=16, sparsity=0.5, threads=None):
+    """The same greedy loop with the dense-masked PyTorch CATS MLP in fp32 on the host cores, on a reduced model
+    (num_layers of the 32 layers, a short prompt, gen_len tokens); the per-token time is scaled to 32 layers."""
+    if threads:
+        torch.set_num_threads(threads)
+    cfg = DecoderConfig(num_layers=num_layers, max_len=prompt_len + gen_len)
+    model = LlamaDecoder(cfg, torch.float32, "cpu", seed=0).eval()
+    model.calibrate(sparsity, n_seq=2, seq_len=prompt_len, chunk=2)
+    model.set_mlp_mode("cats_torch")
+    g = torch.Generator().manual_seed(7)
+    prompt = torch.randint(0, cfg.vocab_size, (1, prompt_len), generator=g)
+    model.reset_cache(1)
+    logits = model.forward(prompt, torch.arange(prompt_len))
+    tok = logits[:, -1].argmax(-1, keepdim=True)
+    t0 = time.perf_counter()
+    for i in range(gen_len - 1):
+        logits = model.forward(tok, torch.tensor([prompt_len + i]))
+        tok = logits[:, -1].argmax(-1, keepdim=True)
+    per_tok = (time.perf_counter() - t0) / (gen_len - 1)
+    lm_head = 0.0  # lm_head + embedding are included once in per_tok; scale only the layer part
+    return {"tok_s_32_layers_extrapolated": round(1.0 / (per_tok * 32 / num_layers), 3), "measured_layers": num_layers,
+            "measured_tokens": gen_len - 1, "ms_per_token_measured": round(per_tok * 1e3, 2), "threads": torch.get_num_threads()}

@@ -1,0 +1,188 @@
+"""GPU tests of the drop-in boundary above the C ABI: every torch.ops.flash_gemv op and Python composite of the
+reference package, the CatsMLP module switches and the graph-replayed decode loop, against the CPU oracle."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from tests.util import TOL, calibrate, dev, make_mlp
+
+pytestmark = pytest.mark.gpu
+
+fg = None
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _load():
+    global fg
+    assert torch.cuda.is_available()
+    import flash_gemv
+
+    fg = flash_gemv
+
+
+def close(got, want, dtype):
+    tol = dict(TOL[dtype])
+    tol["atol"] *= max(1.0, float(want.float().abs().max()))
+    torch.testing.assert_close(got.detach().cpu().float().reshape(want.shape), want.float(), **tol)
+
+
+CASES = [(512, 1024, 1, torch.float16), (1024, 1536, 2, torch.bfloat16), (256, 512, 2, torch.float32), (4096, 2048, 1, torch.float16)]
+
+
+@pytest.mark.parametrize("H,I,B,dtype", CASES)
+def test_reference_ops(oracle, H, I, B, dtype):
+    m = make_mlp(H, I, B, dtype, seed=H + I + B)
+    t = calibrate(m["wg"], [0.5])[0]
+    d = dev(m)
+    x3 = d["x"].view(B, 1, H)
+    ref = oracle.c_mlp(m["x"], m["wg"], m["wu"], m["wd"], t)
+
+    # gate + flag family (output / flag are written in full: garbage-filled buffers on purpose)
+    for op in (fg.fuse_gemv_flag, fg.fuse_gemv_flag_batch, fg.fuse_gemv_flag_local):
+        a = torch.full((B, 1, I), 7.0, dtype=dtype, device="cuda")
+        flag = torch.ones(B, 1, I, dtype=torch.bool, device="cuda")
+        op(x3, d["wg"], a, flag, t)
+        assert torch.equal(flag, torch.abs(a) > t)
+        torch.testing.assert_close(a.cpu().float().view(B, I), ref["a"].float(), rtol=2e-2, atol=2e-3)
+    same = oracle.c_mlp(m["x"], m["wg"], m["wu"], m["wd"], t, a_in=a.cpu().view(B, I), flag_in=flag.cpu().view(B, I))
+
+    # sparse up in place, then sparse down into a pre-zeroed fp32 buffer (the reference's three-call sequence)
+    z = a.clone()
+    fg.fuse_flag_gemv_local(x3, d["wu"], z, flag)
+    close(z, same["z"], dtype)
+    y32 = torch.zeros(B, 1, H, dtype=torch.float32, device="cuda")
+    fg.atomic_gemv(z, d["wdt"], y32, flag)
+    close(y32, same["y"], dtype)
+
+    # gate + up in one op
+    out = torch.empty(B, 1, I, dtype=dtype, device="cuda")
+    flag2 = torch.zeros(B, 1, I, dtype=torch.bool, device="cuda")
+    fg.fuse_gemv_flag_gemv(x3, d["wg"], d["wu"], out, flag2, t)
+    assert torch.equal(flag2, flag)
+    close(out, same["z"], dtype)
+
+    # whole-MLP ops, neuron-major down, fp32 accumulate
+    for op, with_flag in ((fg.fuse_gemv_gemv_gemv, False), (fg.flag_gemv_gemv_atomic, False), (fg.fuse_gemv_flag_gemv_gemv, True)):
+        y32 = torch.zeros(B, 1, H, dtype=torch.float32, device="cuda")
+        if with_flag:
+            f3 = torch.zeros(B, 1, I, dtype=torch.bool, device="cuda")
+            op(x3, d["wg"], d["wu"], d["wdt"], y32, f3, t)
+            assert torch.equal(f3, flag)
+        else:
+            op(x3, d["wg"], d["wu"], d["wdt"], y32, t)
+        close(y32, same["y"], dtype)
+
+    # whole-MLP ops, HF-layout down
+    y = torch.empty(B, 1, H, dtype=dtype, device="cuda")
+    fg.flag_gemv_gemv(x3, d["wg"], d["wu"], d["wd"], y, t)
+    close(y, same["y"], dtype)
+    inner = {torch.float16: fg.flag_gemv_gemv_inner, torch.float32: fg.flag_gemv_gemv_inner_fp32, torch.bfloat16: fg.flag_gemv_gemv_inner_bf16}[dtype]
+    y = inner(x3, d["wg"], d["wu"], d["wd"], t)
+    assert y.shape == x3.shape and y.dtype == dtype
+    close(y, same["y"], dtype)
+    y2 = inner(d["x"], d["wg"], d["wu"], d["wd"], t)          # 2-D input, as the reference allows
+    assert y2.shape == d["x"].shape
+    wrong = {torch.float16: fg.flag_gemv_gemv_inner_bf16, torch.float32: fg.flag_gemv_gemv_inner, torch.bfloat16: fg.flag_gemv_gemv_inner_fp32}[dtype]
+    with pytest.raises(RuntimeError):
+        wrong(x3, d["wg"], d["wu"], d["wd"], t)
+
+    # Python composites.  Gate weight is (H, I) there and x_1 comes from torch, so flags follow torch's gate values.
+    wg_t = d["wg"].t().contiguous()
+    x_1 = F.silu(torch.matmul(x3, wg_t))
+    flags_t = torch.abs(x_1) > t
+    same_t = oracle.c_mlp(m["x"], m["wg"], m["wu"], m["wd"], t, a_in=x_1.cpu().view(B, I), flag_in=flags_t.cpu().view(B, I))
+    y = fg.gemv_gemv_triton(x3, x_1, d["wu"], d["wdt"], t)
+    assert y.shape == (B, 1, H) and y.dtype == dtype
+    close(y, same_t["y"], dtype)
+    close(fg.flag_gemv_gemv_triton(x3, wg_t, d["wu"], d["wdt"], t), same_t["y"], dtype)
+    zt = fg.gather_gemv_elemul_flag_3d(x3, x_1, d["wu"], flags_t)
+    close(zt, same_t["z"], dtype)
+    close(fg.gather_transposed_gemv_flag_3d(zt, d["wdt"], flags_t), same_t["y"], dtype)
+    close(fg.cats_mlp(x3, d["wg"], d["wu"], d["wdt"], t), same["y"], dtype)
+    ys, fl, cnt = fg.cats_mlp_stats(x3, d["wg"], d["wu"], d["wdt"], t)
+    assert torch.equal(fl.view(B, 1, I), flag) and int(cnt) == int(flag.view(B, I).any(0).sum())
+    if B == 1:  # index-list (DejaVu-style) composites take a 2-D single row
+        close(fg.flag_gemv_gemv_dejavu(d["x"], wg_t, d["wu"], d["wdt"], t), same_t["y"], dtype)
+        close(fg.flag_gemv_gemv_fuse_dejavu(d["x"], wg_t, d["wu"], d["wdt"], t), same_t["y"], dtype)
+
+
+def test_fuse_gemv_cmp_compact_list(oracle):
+    m = make_mlp(4096, 14336, 1, torch.float16, seed=0, dist="uniform")   # the one shape the reference op accepts
+    d = dev(m)
+    x3 = d["x"].view(1, 1, 4096)
+    out = torch.zeros(1, 1, 14336, dtype=torch.float16, device="cuda")
+    idx = torch.zeros(14336, dtype=torch.int64, device="cuda")
+    n = fg.fuse_gemv_cmp(x3, d["wg"], out, idx, 0.2)
+    a = torch.empty(1, 1, 14336, dtype=torch.float16, device="cuda")
+    flag = torch.empty(14336, dtype=torch.bool, device="cuda")
+    fg.fuse_gemv_flag(x3, d["wg"], a, flag, 0.2)
+    want_idx, want_n = oracle.c_compact(flag)
+    assert n == want_n
+    assert torch.equal(idx[:n].cpu(), want_idx)
+    assert torch.equal(out.flatten()[:n].cpu(), a.flatten().cpu()[want_idx])
+
+
+def test_bad_arguments_raise_not_exit():
+    x = torch.zeros(9, 1, 64, dtype=torch.float16, device="cuda")
+    w = torch.zeros(96, 64, dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="batch"):
+        fg.cats_mlp(x, w, w, w, 0.1)
+    with pytest.raises(RuntimeError, match="must be"):
+        fg.cats_mlp(x[:1], w, w[:, :32].contiguous(), w, 0.1)
+    with pytest.raises(RuntimeError, match="dtype"):
+        fg.cats_mlp(x[:1], w, w.float(), w, 0.1)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        fg.cats_mlp(x[:1], w, w, torch.zeros(64, 96, dtype=torch.float16, device="cuda").t(), 0.1)
+
+
+def test_cats_mlp_module_methods_agree(oracle):
+    from cats_amd.mlp import CatsMLP
+
+    torch.manual_seed(0)
+    for dtype in (torch.float16, torch.bfloat16, torch.float32):
+        mod = CatsMLP(512, 1024, dtype=dtype, device="cuda")
+        with torch.no_grad():
+            for p in mod.parameters():
+                p.copy_((torch.randn(p.shape, device="cuda") * 0.05).to(dtype))
+        x = torch.randn(2, 1, 512, device="cuda").to(dtype)
+        with torch.no_grad():   # threshold in the widest gap near the median, so no activation sits on the knife edge
+            mags = F.silu(mod.gate_proj(x)).abs().float().flatten().sort().values
+        mid = mags.numel() // 2
+        gaps = mags[mid - 20:mid + 20].diff()
+        j = int(gaps.argmax())
+        mod.dead_threshold = float((mags[mid - 20 + j] + mags[mid - 20 + j + 1]) / 2)
+        mod.is_profile, mod.sp_method = True, 0
+        with torch.no_grad():
+            want = mod(x)
+        for method in (1, 2, 3):
+            mod.prepare_decode(method)
+            with torch.no_grad():
+                got = mod(x)
+            assert got.shape == want.shape and got.dtype == dtype
+            torch.testing.assert_close(got.float(), want.float(), **TOL[dtype])
+        xp = torch.randn(1, 7, 512, device="cuda").to(dtype)       # prefill stays on the dense-masked branch
+        mod.sp_method = 0
+        with torch.no_grad():
+            wantp = mod(xp)
+            mod.prepare_decode(3)
+            torch.testing.assert_close(mod(xp), wantp)
+
+
+def test_decode_loop_graph_replay_matches_eager():
+    from cats_amd import decoder as dec
+
+    cfg = dec.DecoderConfig(hidden_size=256, intermediate_size=512, num_layers=3, num_heads=4, vocab_size=503, max_len=64)
+    model = dec.LlamaDecoder(cfg, torch.float16, "cuda", seed=0, init_std=0.05).eval()
+    model.calibrate(0.5, n_seq=4, seq_len=16, chunk=4)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    prompt = torch.randint(0, 503, (1, 12), generator=g, device="cuda")
+    model.set_mlp_mode("cats")
+    eager, _ = model.generate_greedy(prompt, 24, use_graph=False)
+    for _ in range(2):   # replayed graphs must keep giving the eager tokens
+        graphed, secs = model.generate_greedy(prompt, 24, use_graph=True)
+        assert torch.equal(eager, graphed) and secs > 0
+    # the HIP path and the dense-masked PyTorch path pick the same tokens (identical masks up to rounding ties)
+    model.set_mlp_mode("cats_torch")
+    torch_tokens, _ = model.generate_greedy(prompt, 24, use_graph=False)
+    agree = float((torch_tokens == eager).float().mean())
+    assert agree >= 0.9, f"only {agree:.2f} of the greedy tokens agree between the HIP and PyTorch CATS paths"
