@@ -26,6 +26,9 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+# HBM bytes per launch of the gate+up kernel at 50 % sparsity, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a
+# 256 MiB copy (profiles/cats_mlp_llama7b_fp16_b1_s50_hbm_counters.md): 132603 KiB read + 54 KiB written.
+MEASURED_HBM_BYTES_GATE_UP = int((132603 + 54) * 1024)
 H, I = 4096, 11008
 SPARSITIES = [0.0, 0.3, 0.5, 0.7, 0.9]
 
@@ -54,6 +57,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="time plain stream launches only")
     ap.add_argument("--decode", action="store_true", help="also run the 32-layer decode loop (config 5)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run one 256 MiB device-to-device copy first: a kernel of known traffic for scaling rocprof counters")
     ap.add_argument("--down-groups", type=int, default=0)
     ap.add_argument("--down-block", type=int, default=0)
     args = ap.parse_args()
@@ -72,6 +77,14 @@ def main():
     torch.cuda.set_device(dev)
     dtype, sz, B = torch.float16, 2, 1
     capi.set_tuning(0, args.down_groups, args.down_block, 0)
+
+    if args.copy_calibration:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- synthetic layer sets --------------------------------------------------------------------------------
     g = torch.Generator(device="cuda").manual_seed(0)
@@ -222,7 +235,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(b_gu / us_gate_up * 1e-3 / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_HBM_BYTES_GATE_UP if abs(args.sparsity - 0.5) < 1e-9 else None,
             "bytes_per_launch": int(b_gu),
             "us_per_launch": round(us_gate_up, 3),
             "second_kernel": {"kernel": "cats::down_kernel<F16,B=1> (sparse neuron-major down)", "bytes_per_launch": int(b_dn),
