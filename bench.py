@@ -59,6 +59,7 @@ def main():
     ap.add_argument("--decode", action="store_true", help="also run the 32-layer decode loop (config 5)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run one 256 MiB device-to-device copy first: a kernel of known traffic for scaling rocprof counters")
+    ap.add_argument("--gate-variant", type=int, default=0)
     ap.add_argument("--down-groups", type=int, default=0)
     ap.add_argument("--down-block", type=int, default=0)
     args = ap.parse_args()
@@ -76,7 +77,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     dtype, sz, B = torch.float16, 2, 1
-    capi.set_tuning(0, args.down_groups, args.down_block, 0)
+    capi.set_tuning(args.gate_variant, args.down_groups, args.down_block, 0)
 
     if args.copy_calibration:
         src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
@@ -135,12 +136,12 @@ def main():
         return e0.elapsed_time(e1) * 1e3 / steps  # us per step
 
     def time_cats(t, steps, warmup, stages=0):
-        capi.set_tuning(0, args.down_groups, args.down_block, stages)
+        capi.set_tuning(args.gate_variant, args.down_groups, args.down_block, stages)
         prepared = [mlp_args(st, t) for st in sets]
         n = len(prepared)
         fn = L.cats_mlp
         us = time_region(lambda i: fn(*prepared[i % n]), steps, warmup)
-        capi.set_tuning(0, args.down_groups, args.down_block, 0)
+        capi.set_tuning(args.gate_variant, args.down_groups, args.down_block, 0)
         return us
 
     def time_cats_graph(t, steps, warmup):

@@ -16,7 +16,6 @@ template <> hipError_t launch_rows<F32>(int, int, const RowsArgs&, hipStream_t);
 template <> hipError_t launch_down<F16>(int, bool, const DownArgs&, int, hipStream_t);
 template <> hipError_t launch_down<BF16>(int, bool, const DownArgs&, int, hipStream_t);
 template <> hipError_t launch_down<F32>(int, bool, const DownArgs&, int, hipStream_t);
-
 namespace {
 
 Tuning g_tuning = {0, 0, 0, 0};
@@ -26,7 +25,7 @@ long long* g_tbuf_down = nullptr;
 #endif
 
 constexpr int kMaxSlabs = 128;
-constexpr size_t kCounterBytes = 1024;  // done[128] | arrive | pad
+constexpr size_t kCounterBytes = 1024;  // uint32 words: done[0..127] | arrive 128 | count 192
 
 __global__ void fill_zero_kernel(u32x4* p, size_t n16) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) p[i] = zero4();
@@ -162,6 +161,7 @@ void fill_rows(RowsArgs& a, const void* x, const void* w, int K, int N, int nb, 
 
 int do_rows(int mode, int dtype, const RowsArgs& a_in, hipStream_t s) {
   RowsArgs a = a_in;
+  if (g_tuning.gate_variant > 0) a.lds_floor = (160 * 1024) / g_tuning.gate_variant - 1024;  // at most gate_variant workgroups per CU
 #ifdef CATS_TIMING
   a.tbuf = g_tbuf_rows;
 #endif

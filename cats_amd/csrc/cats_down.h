@@ -62,7 +62,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction; say so
   const int nwaves = blockDim.x >> 6;
   const int slab = blockIdx.x % p.nslab;
   const int group = blockIdx.x / p.nslab;

@@ -23,7 +23,8 @@ hipError_t launch_rows_one(const RowsArgs& a, hipStream_t stream) {
   auto kern = rows_kernel<DT, B, kR, kCB, FULL, MODE, XLDS, WAVES>;
   const int rows_per_block = WAVES * kR;
   const int grid = (a.N + rows_per_block - 1) / rows_per_block;
-  const size_t lds = XLDS ? (size_t)B * ((a.nch + kCB - 1) / kCB * kCB) * kWave * sizeof(u32x4) : 0;
+  size_t lds = XLDS ? (size_t)B * ((a.nch + kCB - 1) / kCB * kCB) * kWave * sizeof(u32x4) : 0;
+  if ((size_t)a.lds_floor > lds) lds = (size_t)a.lds_floor;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;

@@ -8,7 +8,7 @@
 namespace cats {
 
 struct Tuning {
-  int gate_variant;  // reserved for alternative gate kernels; 0 = default
+  int gate_variant;  // N > 0: cap the rows kernel at N workgroups per CU (dynamic-LDS floor); 0 = no cap
   int down_groups;   // 0 = default (about one workgroup per CU over all slabs)
   int down_block;    // 0 = default (1024 threads)
   int stages;        // cats_mlp only: 0 = both launches, 1 = gate+up only, 2 = down only (profiling)

@@ -38,6 +38,7 @@ struct RowsArgs {
   int nch;               // 64-lane vector chunks per row: ceil(K / (64 * VEC))
   int row_vecs;          // K / VEC
   float t;               // threshold, already rounded through dtype
+  int lds_floor;         // host side only: request at least this much dynamic LDS (caps workgroups per CU); 0 = none
 #ifdef CATS_TIMING
   long long* tbuf;       // [gridDim][8] wall-clock stamps (100 MHz) at phase boundaries, development builds only
 #endif
@@ -65,6 +66,10 @@ __device__ __forceinline__ void rows_issue(const u32x4* __restrict__ w, const in
         const int v = (c0 + cc) * kWave + lane;
         wv[r][cc] = load_stream(wr + (FULL ? v : min(v, vlast)));
       }
+    } else {
+      // defined on every path: inside a persistent loop an undefined value would stay live across iterations
+#pragma unroll
+      for (int cc = 0; cc < CB; cc++) wv[r][cc] = zero4();
     }
   }
 }
@@ -110,8 +115,11 @@ __device__ __forceinline__ void rows_dot(const u32x4* __restrict__ w, const int 
     }
 }
 
+// B == 1 asks for 6 waves per SIMD (80 VGPRs): 6 workgroups of 4 waves per CU hold all 1376 workgroups of an
+// 11008-row matrix at once, so no workgroup starts late and runs its two dependent passes on a draining machine.
 template <class DT, int B, int R, int CB, bool FULL, int MODE, bool XLDS, int WAVES>
-__global__ __launch_bounds__(WAVES* kWave) void rows_kernel(RowsArgs p) {
+__global__ __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_eu(B == 1 && WAVES == 4 && FULL ? 6 : 1, 8)))
+void rows_kernel(RowsArgs p) {
   typedef typename DT::st st;
   extern __shared__ u32x4 xs[];  // [B][round_up(nch, CB) * 64] vectors (XLDS only)
   __shared__ uint32_t s_maskbits;
@@ -119,7 +127,7 @@ __global__ __launch_bounds__(WAVES* kWave) void rows_kernel(RowsArgs p) {
   __shared__ int s_wtot[WAVES];
 
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform by construction; say so
   constexpr int kThreads = WAVES * kWave;
   constexpr int kRowsPerBlock = WAVES * R;
   static_assert(kRowsPerBlock % 8 == 0 && kRowsPerBlock <= 32, "mask bytes are assembled in one 32-bit LDS word");

@@ -129,7 +129,9 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
 int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out,
                            int B, int H, int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream);
 
-/* Launch-shape knobs for experiments and profiling; 0 keeps the built-in choice.  `stages` restricts cats_mlp
+/* Launch-shape knobs for experiments and profiling; 0 keeps the built-in choice.  gate_variant N > 0 caps the
+ * gate / up kernel at N resident workgroups per CU; down_groups / down_block set the neuron groups and the
+ * workgroup size of the sparse down kernel.  `stages` restricts cats_mlp
  * to one of its two launches (1 = gate+up only, 2 = sparse down only, over whatever mask and z the workspace
  * holds from the previous full call) so each kernel can be timed alone.  Process-global; not in the reference. */
 int cats_set_tuning(int gate_variant, int down_groups, int down_block, int stages);
