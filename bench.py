@@ -55,6 +55,7 @@ def main():
     ap.add_argument("--sparsity", type=float, default=0.5)
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the Mistral bf16 and batch 2/4/8 configurations")
     ap.add_argument("--no-graph", action="store_true", help="time plain stream launches only")
     ap.add_argument("--decode", action="store_true", help="also run the 32-layer decode loop (config 5)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -247,6 +248,11 @@ def main():
         "sweep": sweep,
     }
 
+    if not args.no_extra:
+        del sets
+        torch.cuda.empty_cache()
+        out["other_configs"] = other_configs(torch, F, capi, L, max(200, args.steps // 4), max(50, args.warmup // 4))
+
     if args.decode:
         from cats_amd import decoder
 
@@ -256,6 +262,75 @@ def main():
         out["cpu_baseline"] = cpu_baseline(torch, F, thr[0.5] if 0.5 in thr else t50)
 
     print(json.dumps(out))
+
+
+def other_configs(torch, F, capi, L, steps, warmup):
+    """The remaining single-layer configurations: Mistral-7B shape in bf16 with heavy-tailed gate rows (50 / 70 %), and
+    the Llama fp16 layer at batch 2 / 4 / 8 with pairwise-correlated rows (per-row masks, union gathering)."""
+    import math
+
+    dev = torch.device("cuda:0")
+    res = []
+
+    def run(name, Hh, Ii, B, dtype, code, sparsities, heavy_tail=False, corr=0.0, nsets=6):
+        g = torch.Generator(device="cuda").manual_seed(1)
+        sz = 2
+        sets = []
+        for _ in range(nsets):
+            wg = torch.randn(Ii, Hh, generator=g, device=dev) * 0.02
+            if heavy_tail:
+                wg = wg * torch.exp(torch.randn(Ii, 1, generator=g, device=dev) * 0.5)
+            wu = torch.randn(Ii, Hh, generator=g, device=dev) * 0.02
+            wd = torch.randn(Hh, Ii, generator=g, device=dev) * 0.02
+            sets.append(dict(wg=wg.to(dtype), wu=wu.to(dtype), wd=wd.to(dtype), wdt=wd.to(dtype).t().contiguous()))
+            del wg, wu, wd
+        if corr > 0:
+            x = (math.sqrt(corr) * torch.randn(1, Hh, generator=g, device=dev) + math.sqrt(1 - corr) * torch.randn(B, Hh, generator=g, device=dev)).to(dtype)
+        else:
+            x = torch.randn(B, Hh, generator=g, device=dev).to(dtype)
+        X = torch.randn(256, Hh, generator=g, device=dev)
+        act = F.silu(X @ sets[0]["wg"].float().t()).abs().flatten().cpu()
+        ws = capi.Workspace(B, Hh, Ii)
+        y = torch.empty(B, Hh, dtype=dtype, device=dev)
+        count = torch.zeros(1, dtype=torch.int32, device=dev)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        p = lambda t: ctypes.c_void_p(t.data_ptr())
+
+        def timed(fn):
+            for i in range(warmup):
+                fn(i)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(steps):
+                fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / steps
+
+        us_dense = timed(lambda i: F.linear(F.silu(F.linear(x, sets[i % nsets]["wg"])) * F.linear(x, sets[i % nsets]["wu"]), sets[i % nsets]["wd"]))
+        for s in sparsities:
+            t = float(torch.kthvalue(act, max(1, int(round(s * act.numel())))).values)
+            ks = []
+            for st in sets:
+                capi.check(L.cats_mlp(p(x), p(st["wg"]), p(st["wu"]), p(st["wdt"]), p(y), None, None, p(count), B, Hh, Ii, code, ctypes.c_float(t),
+                                      p(ws.buf), ws.nbytes, stream), "cats_mlp")
+                ks.append(int(count.item()))
+            k = sum(ks) / len(ks)
+            prepared = [(p(x), p(st["wg"]), p(st["wu"]), p(st["wdt"]), p(y), None, None, None, B, Hh, Ii, code, ctypes.c_float(t), p(ws.buf), ws.nbytes, stream)
+                        for st in sets]
+            us = timed(lambda i: L.cats_mlp(*prepared[i % nsets]))
+            tb = sz * Hh * Ii + 2 * sz * Hh * k + sz * B * (2 * Hh + Ii) + 4 * k + 4
+            res.append(dict(config=name, batch=B, row_sparsity_target=s, union_sparsity=round(1 - k / Ii, 4), us=round(us, 2),
+                            touched_MB=round(tb / 1e6, 1), GBps=round(tb / us * 1e-3, 1), hbm_frac=round(tb / us * 1e-3 / HBM_PEAK_GBPS, 4),
+                            dense_us=round(us_dense, 2), speedup_vs_dense=round(us_dense / us, 3)))
+        del sets
+        torch.cuda.empty_cache()
+
+    run("mistral7b_bf16_heavy_tail", 4096, 14336, 1, torch.bfloat16, capi.BF16, [0.5, 0.7], heavy_tail=True)
+    for B in (2, 4, 8):
+        run(f"llama7b_fp16_batch{B}_corr0.5", 4096, 11008, B, torch.float16, capi.F16, [0.5], corr=0.5)
+    return res
 
 
 def cpu_baseline(torch, F, t):

@@ -15,7 +15,7 @@ constexpr int kCB = 8;   // 64-lane chunks whose loads are issued together: 8 x 
 constexpr int kDownU = 8;  // rows in flight per lane in the down kernel
 
 // Workgroup width by batch: x is staged per workgroup, so wider batches share it across more waves.
-template <int B> struct WavesFor { static constexpr int value = B <= 2 ? 4 : (B == 4 ? 8 : 16); };
+template <int B> struct WavesFor { static constexpr int value = B <= 2 ? 4 : 8; };
 
 template <class DT, int B, bool FULL, int MODE, bool XLDS>
 hipError_t launch_rows_one(const RowsArgs& a, hipStream_t stream) {

@@ -146,7 +146,9 @@ void rows_kernel(RowsArgs p) {
   // first block of weight loads, and only the x values are waited for before the LDS writes and the barrier --
   // the weight loads stay in flight across both.
   u32x4 wv[R][CB];
-  constexpr int kXPre = 2;  // x vectors per thread fetched ahead of the weights (covers B*H*sizeof <= 8 KiB per 256 threads)
+  // x vectors per thread fetched ahead of the weights: all of x for H = 4096 in 16-bit types (B * 512 vectors)
+  constexpr int kXPreAll = (B * 512 + kThreads - 1) / kThreads;
+  constexpr int kXPre = kXPreAll < 4 ? kXPreAll : 4;  // more would spill at B = 8
   const int nchv = (p.nch + CB - 1) / CB * CB * kWave;  // padded vectors per x row
   u32x4 xpre[kXPre];
   if (XLDS) {
