@@ -193,7 +193,7 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   int block = g_tuning.down_block > 0 ? g_tuning.down_block : 1024;
   if (block < 128) block = 128;  // wave 0 builds the index list, the others stage z
   if (block > 1024) block = 1024;
-  block = block / 64 * 64;
+  while (block & (block - 1)) block &= block - 1;  // the fold across waves halves their number per round
   const int bt = batch_template(B);
   // about one workgroup per CU over all slabs; more groups if a group's list and z would not fit in LDS
   int ngroup = g_tuning.down_groups > 0 ? g_tuning.down_groups : 256 / d.nslab;

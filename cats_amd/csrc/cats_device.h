@@ -34,6 +34,7 @@ __device__ __forceinline__ u32x4 zero4() {
 // fromf   float -> storage, round to nearest even
 // rnd     float -> float, rounded through the storage type
 // dot     acc + sum over the VEC element pairs of two vectors, accumulated in fp32
+// dot2    (16-bit types) acc + the two products of one packed pair
 // axpy    acc[i] += z * w[i] for the VEC elements of one vector
 
 struct F16 {
@@ -47,6 +48,9 @@ struct F16 {
     for (int i = 0; i < 4; i++)
       acc = __builtin_amdgcn_fdot2(as_f16x2(w[i]), as_f16x2(x[i]), acc, false);
     return acc;
+  }
+  static __device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {
+    return __builtin_amdgcn_fdot2(as_f16x2(w), as_f16x2(x), acc, false);
   }
   static __device__ __forceinline__ void axpy(u32x4 w, float z, float* acc) {
 #pragma unroll
@@ -74,6 +78,9 @@ struct BF16 {
     for (int i = 0; i < 4; i++)
       acc = __builtin_amdgcn_fdot2_f32_bf16(as_bf16x2(w[i]), as_bf16x2(x[i]), acc, false);
     return acc;
+  }
+  static __device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(as_bf16x2(w), as_bf16x2(x), acc, false);
   }
   static __device__ __forceinline__ void axpy(u32x4 w, float z, float* acc) {
 #pragma unroll

@@ -47,23 +47,64 @@ struct DownArgs {
 #define CATS_STAMP(slot) do { } while (0)
 #endif
 
+// Adds z-weighted weight vectors of two active rows into acc[b][0..VEC).  16-bit types interleave the two rows
+// element-wise (one v_perm per dword) so that one v_dot2 per column does both rows; fp32 is two plain axpy.
+template <class DT, int B>
+struct PairAxpy {
+  typedef typename DT::st st;
+  static __device__ __forceinline__ void run(u32x4 wa, u32x4 wb, const st* za, const st* zb, int zstride, float (*acc)[DT::VEC]) {
+#pragma unroll
+    for (int b = 0; b < B; b++) {
+      DT::axpy(wa, DT::tof(za[b * zstride]), acc[b]);
+      DT::axpy(wb, DT::tof(zb[b * zstride]), acc[b]);
+    }
+  }
+};
+
+template <class DT, int B>
+struct PairAxpy16 {
+  // zp[b] = (z[b, row a], z[b, row b]) packed in storage type; a missing second row has weight and z zero
+  static __device__ __forceinline__ void run(u32x4 wa, u32x4 wb, const uint32_t* zp, float (*acc)[8]) {
+    uint32_t lo[4], hi[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      lo[i] = __builtin_amdgcn_perm(wb[i], wa[i], 0x05040100u);  // (wa[i].lo16, wb[i].lo16): column 2i of both rows
+      hi[i] = __builtin_amdgcn_perm(wb[i], wa[i], 0x07060302u);  // (wa[i].hi16, wb[i].hi16): column 2i + 1
+    }
+#pragma unroll
+    for (int b = 0; b < B; b++) {
+      const uint32_t z2 = zp[b];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        acc[b][2 * i] = DT::dot2(lo[i], z2, acc[b][2 * i]);
+        acc[b][2 * i + 1] = DT::dot2(hi[i], z2, acc[b][2 * i + 1]);
+      }
+    }
+  }
+};
+
 template <class DT, int B, bool ZF32, int U>
 __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   typedef typename DT::st st;
   constexpr int VEC = DT::VEC;
   constexpr int kSlabCols = kWave * VEC;
+  constexpr int UP = U / 2;  // row pairs in flight per lane
+  constexpr bool kPacked = sizeof(st) == 2;  // 16-bit types: z of a row pair travels as one packed dword
   extern __shared__ float s_dyn[];
-  // dynamic LDS: [chunk] int list | [B][chunk] float z (indexed by j - j0) | [nwaves][64*VEC] float partials
+  // dynamic LDS, streaming phase: [chunk] int list | [B][chunk] z in storage type (indexed by j - j0)
+  //                               | 16-bit types: [chunk / 2][B] packed z pairs in list order
+  // afterwards reused for the fold: [nwaves / 2][B][VEC][64] float
   int* s_list = (int*)s_dyn;
-  float* s_z = s_dyn + p.chunk;
-  float* s_red = s_z + (size_t)B * p.chunk;
+  st* s_z = (st*)(s_dyn + p.chunk);
+  uint32_t* s_zp = (uint32_t*)(s_dyn + p.chunk) + (B * p.chunk * sizeof(st) + 3) / 4;
+  float* s_red = s_dyn;
   __shared__ int s_n;
   __shared__ int s_last;
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction; say so
-  const int nwaves = blockDim.x >> 6;
+  const int nwaves = blockDim.x >> 6;                         // a power of two
   const int slab = blockIdx.x % p.nslab;
   const int group = blockIdx.x / p.nslab;
   const int j0 = group * p.chunk;
@@ -92,23 +133,30 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
     }
     if (lane == 0) s_n = base;
   } else {
+    // one flat loop over (b, q) so that the loads of all batch rows are in flight together
     const int span = j1 - j0;
-    for (int b = 0; b < B; b++) {
-      for (int q = tid - kWave; q < span; q += blockDim.x - kWave) {
-        float zv = 0.f;
-        if (b < p.nb) {
-          const size_t o = (size_t)b * p.I + j0 + q;
-          zv = ZF32 ? ((const float*)p.z)[o] : DT::tof(((const st*)p.z)[o]);
-        }
-        s_z[b * p.chunk + q] = zv;
-      }
+    const int total = p.nb * span;
+    for (int i = tid - kWave; i < total; i += blockDim.x - kWave) {
+      const int b = i / span, q = i - b * span;
+      const size_t o = (size_t)b * p.I + j0 + q;
+      s_z[b * p.chunk + q] = ZF32 ? DT::fromf(((const float*)p.z)[o]) : ((const st*)p.z)[o];
     }
+    for (int i = p.nb * p.chunk + tid - kWave; i < B * p.chunk; i += blockDim.x - kWave) s_z[i] = DT::fromf(0.f);
   }
   __syncthreads();
   const int n = s_n;
+  const int nfull = n >> 1;  // whole pairs; pair k is list entries 2k and 2k + 1
+  if (kPacked) {
+    for (int i = tid; i < nfull * B; i += blockDim.x) {
+      const int k = i / B, b = i - k * B;
+      const uint32_t za = s_z[b * p.chunk + s_list[2 * k] - j0], zb = s_z[b * p.chunk + s_list[2 * k + 1] - j0];
+      s_zp[i] = za | (zb << 16);
+    }
+    __syncthreads();
+  }
   CATS_STAMP(1);
 
-  // ---- 2. stream the slab segments of the active rows ---------------------------------------------------
+  // ---- 2. stream the slab segments of the active rows, two rows at a time --------------------------------
   float acc[B][VEC];
 #pragma unroll
   for (int b = 0; b < B; b++)
@@ -118,52 +166,82 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   // Lanes past the end of a row (H not a multiple of 64 * VEC) re-read the row's last vector; their sums
   // are dropped at the column check below, so no load is predicated per lane.
   const int v = min(slab * kWave + lane, p.row_vecs - 1);
-  // This wave owns list entries wave, wave + nwaves, ...; split them into passes of at most U, evenly.
-  const int mine = n > wave ? (n - wave + nwaves - 1) / nwaves : 0;
-  const int passes = (mine + U - 1) / U;
+  // This wave owns pairs wave, wave + nwaves, ...; split them into passes of at most UP, evenly.
+  const int mine = nfull > wave ? (nfull - wave + nwaves - 1) / nwaves : 0;
+  const int passes = (mine + UP - 1) / UP;
   const int per = passes ? (mine + passes - 1) / passes : 0;
   for (int t0 = 0; t0 < mine; t0 += per) {
     const int cnt = min(per, mine - t0);  // wave-uniform
-    u32x4 wv[U];
-    int jj[U];
+    u32x4 wa[UP], wb[UP];
+    int kk[UP], ja[UP], jb[UP];
 #pragma unroll
-    for (int u = 0; u < U; u++) {
+    for (int u = 0; u < UP; u++) {
       if (u < cnt) {
-        jj[u] = s_list[wave + (t0 + u) * nwaves];
-        wv[u] = load_stream(p.wd + (size_t)jj[u] * p.row_vecs + v);
+        kk[u] = wave + (t0 + u) * nwaves;
+        ja[u] = __builtin_amdgcn_readfirstlane(s_list[2 * kk[u]]);
+        jb[u] = __builtin_amdgcn_readfirstlane(s_list[2 * kk[u] + 1]);
+        wa[u] = load_stream(p.wd + (size_t)ja[u] * p.row_vecs + v);
+        wb[u] = load_stream(p.wd + (size_t)jb[u] * p.row_vecs + v);
       }
     }
 #pragma unroll
-    for (int u = 0; u < U; u++) {
+    for (int u = 0; u < UP; u++) {
       if (u < cnt) {
-#pragma unroll
-        for (int b = 0; b < B; b++) DT::axpy(wv[u], s_z[b * p.chunk + jj[u] - j0], acc[b]);
+        if constexpr (kPacked) PairAxpy16<DT, B>::run(wa[u], wb[u], s_zp + kk[u] * B, acc);
+        else PairAxpy<DT, B>::run(wa[u], wb[u], s_z + (ja[u] - j0), s_z + (jb[u] - j0), p.chunk, acc);
       }
     }
   }
+  if ((n & 1) && wave == nfull % nwaves) {  // odd list: the last row has no partner
+    const int j = __builtin_amdgcn_readfirstlane(s_list[n - 1]);
+    const u32x4 w = load_stream(p.wd + (size_t)j * p.row_vecs + v);
+#pragma unroll
+    for (int b = 0; b < B; b++) DT::axpy(w, DT::tof(s_z[b * p.chunk + j - j0]), acc[b]);
+  }
 
   CATS_STAMP(2);
-  // ---- 3. fold the waves through LDS; slab partial -> scratch (y_out) or atomics (y32) ---------------------
+  // ---- 3. fold the waves pairwise through LDS (upper half writes, lower half adds), log2(nwaves) rounds ------
+  __syncthreads();  // the list and z are dead from here on; their LDS is reused
+  for (int half = nwaves >> 1; half >= 1; half >>= 1) {
+    if (wave >= half && wave < 2 * half) {
+      float* dst = s_red + (size_t)(wave - half) * B * kSlabCols;
+#pragma unroll
+      for (int b = 0; b < B; b++)
+#pragma unroll
+        for (int e = 0; e < VEC; e++) dst[(b * VEC + e) * kWave + lane] = acc[b][e];
+    }
+    __syncthreads();
+    if (wave < half) {
+      const float* src = s_red + (size_t)wave * B * kSlabCols;
+#pragma unroll
+      for (int b = 0; b < B; b++)
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[b][e] += src[(b * VEC + e) * kWave + lane];
+    }
+    __syncthreads();
+  }
+
+  // wave 0 holds the slab partial: lane l, element e is column (slab*64 + l) * VEC + e
   float* mypart = p.partial + ((size_t)slab * p.ngroup + group) * B * kSlabCols;
+  if (wave == 0) {
 #pragma unroll
-  for (int b = 0; b < B; b++) {
-    if (b < p.nb) {  // uniform
-#pragma unroll
-      for (int e = 0; e < VEC; e++) s_red[wave * kSlabCols + e * kWave + lane] = acc[b][e];
-      __syncthreads();
-      for (int c = tid; c < kSlabCols; c += blockDim.x) {
-        // c = e * 64 + l  ->  column (slab*64 + l) * VEC + e
-        float s = 0.f;
-        for (int w = 0; w < nwaves; w++) s += s_red[w * kSlabCols + c];
+    for (int b = 0; b < B; b++) {
+      if (b < p.nb) {  // uniform
         if (p.y_out) {
-          __hip_atomic_store(&mypart[b * kSlabCols + c], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+          for (int e = 0; e < VEC; e += 2) {
+            const uint64_t two = (uint64_t)__float_as_uint(acc[b][e]) | ((uint64_t)__float_as_uint(acc[b][e + 1]) << 32);
+            __hip_atomic_store((uint64_t*)&mypart[((b * VEC + e) >> 1) * (2 * kWave) + 2 * lane], two, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+          }
         } else {
-          const int e = c >> 6, l = c & 63;
-          const int col = (slab * kWave + l) * VEC + e;
-          if (col < p.H && n > 0) unsafeAtomicAdd(&p.y32[(size_t)b * p.H + col], s);
+#pragma unroll
+          for (int e = 0; e < VEC; e++) {
+            const int col = (slab * kWave + lane) * VEC + e;
+            if (col < p.H && n > 0) unsafeAtomicAdd(&p.y32[(size_t)b * p.H + col], acc[b][e]);
+          }
         }
       }
-      __syncthreads();
     }
   }
 
@@ -191,38 +269,48 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   // ---- 4. last workgroup of the slab adds the partials in group order and writes y ---------------------------
   // Ordering without a release / acquire fence pair (at agent scope those write back and invalidate the whole
   // L2 of the XCD, which costs far more than this kernel): partials are written and read with agent-scope
-  // atomic stores / loads, which are coherent across the device by themselves.  Each wave waits until its own
-  // stores have been acknowledged (s_waitcnt vmcnt(0)), the barrier joins the waves, and only then is the slab
-  // counter bumped -- so when a workgroup reads "I am last" every partial of the slab is in place, and the loads
-  // below, issued after that read, see them.
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt / lgkmcnt untouched
-  __syncthreads();
-  CATS_STAMP(4);
-  if (tid == 0) {
-    const uint32_t prev = __hip_atomic_fetch_add(&p.done[slab], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s_last = prev == (uint32_t)p.ngroup - 1u;
+  // atomic stores / loads, which are coherent across the device by themselves.  The storing wave waits until
+  // its stores have been acknowledged (s_waitcnt vmcnt(0)) and only then bumps the slab counter -- so when a
+  // workgroup reads "I am last" every partial of the slab is in place, and the loads below, issued after
+  // that read, see them.
+  if (wave == 0) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt / lgkmcnt untouched
+    CATS_STAMP(4);
+    if (lane == 0) {
+      const uint32_t prev = __hip_atomic_fetch_add(&p.done[slab], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = prev == (uint32_t)p.ngroup - 1u;
+    }
   }
   __syncthreads();
   CATS_STAMP(5);
   if (!s_last) return;
-  const float* slabpart = p.partial + (size_t)slab * p.ngroup * B * kSlabCols;
-  for (int b = 0; b < p.nb; b++) {
-    for (int c = tid; c < kSlabCols; c += blockDim.x) {
-      const int e = c >> 6, l = c & 63;
-      const int col = (slab * kWave + l) * VEC + e;
-      float s = 0.f;
-      for (int g0 = 0; g0 < p.ngroup; g0 += 8) {  // 8 independent loads in flight, added in group order
-        float t[8];
+  const uint64_t* slabpart = (const uint64_t*)(p.partial + (size_t)slab * p.ngroup * B * kSlabCols);
+  constexpr int kPairs = VEC / 2 * kWave;  // 64-bit items per batch row and group
+  constexpr int kInFlight = 16;
+  for (int item = tid; item < p.nb * kPairs; item += blockDim.x) {
+    const int b = item / kPairs, r = item - b * kPairs;
+    const int e = (r >> 6) * 2, l = r & 63;
+    const int col = (slab * kWave + l) * VEC + e;
+    float s0 = 0.f, s1 = 0.f;
+    for (int g0 = 0; g0 < p.ngroup; g0 += kInFlight) {  // independent loads in flight, added in group order
+      uint64_t t[kInFlight];
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-          const int gg = min(g0 + u, p.ngroup - 1);
-          t[u] = __hip_atomic_load(&slabpart[((size_t)gg * B + b) * kSlabCols + c], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-#pragma unroll
-        for (int u = 0; u < 8; u++)
-          if (g0 + u < p.ngroup) s += t[u];
+      for (int u = 0; u < kInFlight; u++) {
+        const int gg = min(g0 + u, p.ngroup - 1);
+        t[u] = __hip_atomic_load(&slabpart[((size_t)gg * B + b) * kPairs + r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-      if (col < p.H) ((st*)p.y_out)[(size_t)b * p.H + col] = DT::fromf(s);
+#pragma unroll
+      for (int u = 0; u < kInFlight; u++) {
+        if (g0 + u < p.ngroup) {
+          s0 += __uint_as_float((uint32_t)t[u]);
+          s1 += __uint_as_float((uint32_t)(t[u] >> 32));
+        }
+      }
+    }
+    if (col < p.H) {
+      st* y = (st*)p.y_out + (size_t)b * p.H + col;
+      y[0] = DT::fromf(s0);
+      y[1] = DT::fromf(s1);
     }
   }
   if (tid == 0) __hip_atomic_store(&p.done[slab], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -61,7 +61,12 @@ template <class DT, int B, bool ZF32>
 hipError_t launch_down_one(const DownArgs& a, int block, hipStream_t stream) {
   auto kern = down_kernel<DT, B, ZF32, kDownU>;
   const int nwaves = block / kWave;
-  const size_t lds = ((size_t)a.chunk * (1 + B) + (size_t)nwaves * kWave * DT::VEC) * sizeof(float);
+  // streaming phase: index list + z of the range; fold phase (same bytes): half the waves' partial sums
+  // (index list, z, and for 16-bit types the packed z pairs)
+  const size_t zbytes = (size_t)B * a.chunk * sizeof(typename DT::st);
+  const size_t lds_stream = (size_t)a.chunk * sizeof(int) + (zbytes + 3) / 4 * 4 + (sizeof(typename DT::st) == 2 ? zbytes + 4 * B : 0);
+  const size_t lds_fold = (size_t)(nwaves / 2) * B * kWave * DT::VEC * sizeof(float);
+  const size_t lds = (lds_stream > lds_fold ? lds_stream : lds_fold) + 64;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
