@@ -161,6 +161,7 @@ void fill_rows(RowsArgs& a, const void* x, const void* w, int K, int N, int nb, 
 
 int do_rows(int mode, int dtype, const RowsArgs& a_in, hipStream_t s) {
   RowsArgs a = a_in;
+  a.mma = g_tuning.gate_variant >= 0;  // gate_variant < 0: keep batches of 2..8 on the wave-per-row kernel
   if (g_tuning.gate_variant > 0) a.lds_floor = (160 * 1024) / g_tuning.gate_variant - 1024;  // at most gate_variant workgroups per CU
 #ifdef CATS_TIMING
   a.tbuf = g_tbuf_rows;

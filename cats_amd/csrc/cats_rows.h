@@ -39,6 +39,7 @@ struct RowsArgs {
   int row_vecs;          // K / VEC
   float t;               // threshold, already rounded through dtype
   int lds_floor;         // host side only: request at least this much dynamic LDS (caps workgroups per CU); 0 = none
+  int mma;               // host side only: kGateUp with 2..8 batch rows may take the matrix-core kernel
 #ifdef CATS_TIMING
   long long* tbuf;       // [gridDim][8] wall-clock stamps (100 MHz) at phase boundaries, development builds only
 #endif

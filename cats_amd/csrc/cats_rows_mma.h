@@ -1,0 +1,210 @@
+// Fused gate + up pass for batches of 2..8 rows in 16-bit types, on the matrix cores.
+//
+// Why not the wave-per-row kernel: with B batch rows every 16-byte weight vector costs 4 * B v_dot2 and B / 2
+// LDS reads of x per lane.  From B = 4 on, that arithmetic plus the LDS traffic takes as long as the HBM stream
+// itself and the three do not overlap inside a wave.  One v_mfma_f32_16x16x32 eats 1 KiB of weights against all
+// batch rows at once, with one 16-byte LDS read per lane, so the kernel goes back to being a weight stream.
+//
+// Tile shape.  The MFMA wants 16 "rows" x 32 k per instruction with 4 lanes per row, i.e. 64 contiguous bytes
+// per weight row per load instruction -- half a cache line, which streams about 25 % slower than whole lines.
+// So a tile is 8 weight rows x 64 k instead: MFMA row m holds weight row m % 8, k half m / 8, and MFMA column n
+// holds batch row n % 8 with the same k half n / 8.  Eight lanes then read 128 contiguous bytes of a row.  The
+// (m < 8, n < 8) and (m >= 8, n >= 8) quadrants of the result are the two halves of the dot products, the other
+// two quadrants pair mismatched halves and are dropped.
+//
+// Work split.  One persistent workgroup per CU: x is staged once in LDS in operand order (one linear 16-byte
+// read per lane per step).  A workgroup owns tiles blockIdx, blockIdx + grid, ...; its waves split K.  Tiles
+// move through a software pipeline, one per round:
+//   round r:  MFMA on the gate rows of tile r (loaded two rounds ago) -> per-wave partial sums to LDS;
+//             gate loads of tile r + 2 go out; wave 0 adds the partials in wave order, applies SiLU and the
+//             threshold and publishes the tile's union bits; up loads of tile r go out for the active rows only
+//             (lanes of inactive rows are masked off, so no bytes move for them); MFMA on the up rows of tile
+//             r - 1 (loaded one round ago) -> partials -> wave 0 writes z = a * up for tile r - 1.
+// So the gate rows of two tiles and the up rows of one are in flight while a fourth tile is being reduced; the
+// only exposed latencies are the first gate load and the last up load.  The two load rings are addressed
+// statically (the loop is unrolled by two): a register that a load in flight will write cannot be moved.
+#pragma once
+#include "cats_rows.h"
+
+namespace cats {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <class DT> struct Mma;
+template <> struct Mma<F16> {
+  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<BF16> {
+  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+
+constexpr int kMmaWaves = 8;
+constexpr int kMmaThreads = kMmaWaves * kWave;
+constexpr int kMmaTileRows = 8;
+constexpr int kMmaPart = 128;    // floats per wave in a partial buffer (the two useful quadrants)
+
+// dynamic LDS: x operands, gate partials, up partials
+inline size_t rows_mma_lds_bytes(int K) {
+  return (size_t)(K / 64) * kWave * sizeof(u32x4) + 2u * kMmaWaves * kMmaPart * sizeof(float);
+}
+// STEPS = 64-element k steps per wave per tile; the row length must be exactly kMmaWaves * STEPS * 64 so that no
+// load or MFMA sits behind a bounds check (control flow around loads in flight makes the compiler wait for them).
+inline int rows_mma_steps(int K) { return K % (kMmaWaves * 64) == 0 ? K / (kMmaWaves * 64) : 0; }
+
+// UP = false is the gate pass alone (activations, flags and union bits out; no up rows, no z).
+template <class DT, int STEPS, bool UP>
+__global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
+  typedef typename DT::st st;
+  extern __shared__ u32x4 xs[];  // [nsteps][64] x operands, then the partial buffers
+  __shared__ uint32_t s_any;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int kMmaSteps = STEPS;
+  constexpr int nsteps = kMmaWaves * STEPS;
+  float* part_g = (float*)(xs + (size_t)nsteps * kWave);
+  float* part_u = part_g + kMmaWaves * kMmaPart;
+
+  const int ntiles = (p.N + kMmaTileRows - 1) / kMmaTileRows;
+  const int grid = gridDim.x;
+  const int my_tiles = ntiles > (int)blockIdx.x ? (ntiles - blockIdx.x + grid - 1) / grid : 0;
+
+  const int s0 = wave * STEPS;  // this wave's first k step
+  // this lane's weight row inside a tile and its 16-byte piece of the 128-byte step
+  const int jl = lane & 7;
+  const int piece = ((lane >> 3) & 1) * 4 + (lane >> 4);
+  // slot of this lane's accumulators in a partial buffer; the two mismatched quadrants are not stored
+  const int ncol = lane & 15;
+  const bool keep = (lane < 32) ? (ncol < 8) : (ncol >= 8);
+  const int slot = (lane >> 5) * 16 + ((lane >> 4) & 1) * 8 + (ncol & 7);
+
+  // Loads of tile number `it` of this workgroup, never predicated: rows past N re-read the last row (their sums
+  // are dropped); lanes with nothing to fetch -- tiles past the end, and with use_any the rows whose union bit is
+  // clear -- read the first bytes of the matrix over and over, which stay in cache and move nothing from HBM.
+  auto issue = [&](const u32x4* __restrict__ w, int it, u32x4 (&dst)[kMmaSteps], bool use_any) {
+    const bool live = it < my_tiles;  // uniform
+    const int tile = live ? blockIdx.x + it * grid : 0;
+    bool mine = live;
+    if (use_any) mine = live && ((s_any >> jl) & 1u);
+    const int row = min(tile * kMmaTileRows + jl, p.N - 1);
+    const u32x4* src = mine ? w + (size_t)row * p.row_vecs + piece + (size_t)s0 * 8 : w + piece;
+    const int stride = mine ? 8 : 0;
+#pragma unroll
+    for (int c = 0; c < kMmaSteps; c++) dst[c] = load_stream(src + c * stride);
+  };
+  auto multiply = [&](const u32x4 (&src)[kMmaSteps], float* part) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < kMmaSteps; c++) acc = Mma<DT>::run(src[c], xs[(s0 + c) * kWave + lane], acc);
+    if (keep) {
+      float* dst = part + wave * kMmaPart + slot;
+#pragma unroll
+      for (int i = 0; i < 4; i++) dst[i * 32] = acc[i];
+    }
+  };
+  // wave 0, one thread per (row j of the tile, batch row b): adds the waves' partials in wave order
+  const int rj = (lane >> 3), rb = lane & 7;
+  auto reduce = [&](const float* part) -> float {
+    const float* src = part + (rj & 3) * 32 + (rj >> 2) * 8 + rb;
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < kMmaWaves; w++) s += src[w * kMmaPart] + src[w * kMmaPart + 16];
+    return s;
+  };
+
+  // wave 0 carries the gate results of the previous tile until its up sums arrive
+  float prev_a = 0.f;
+  bool prev_act = false, prev_valid = false;
+  uint32_t prev_bits = 0u;
+  int prev_row = 0;
+
+  auto round_body = [&](int r, u32x4 (&gcur)[kMmaSteps], u32x4 (&ucur)[kMmaSteps], u32x4 (&uprev)[kMmaSteps]) {
+    multiply(gcur, part_g);
+    issue(p.w, r + 2, gcur, false);
+    __syncthreads();
+    float a = 0.f;
+    bool act = false, valid = false;
+    uint32_t bits8 = 0u;
+    const int tile = blockIdx.x + r * grid;
+    const int row = tile * kMmaTileRows + rj;
+    if (wave == 0 && r < my_tiles) {
+      valid = row < p.N && rb < p.nb;
+      const float gr = DT::rnd(reduce(part_g));
+      a = DT::rnd(gr / (1.f + expf(-gr)));
+      act = valid && fabsf(a) > p.t;
+      const uint64_t bal = __ballot(act);
+#pragma unroll
+      for (int j = 0; j < 8; j++) bits8 |= ((bal >> (8 * j)) & 0xffull) ? (1u << j) : 0u;
+      if (lane == 0) {
+        s_any = bits8;
+        if (p.mask_out) p.mask_out[tile] = (uint8_t)bits8;
+      }
+      if (valid && p.flag_out) p.flag_out[(size_t)rb * p.N + row] = act ? 1 : 0;
+      if (!UP && valid && p.a_out) ((st*)p.a_out)[(size_t)rb * p.N + row] = DT::fromf(a);
+    }
+    __syncthreads();
+    if (!UP) return;
+    issue(p.w2, r, ucur, true);
+    multiply(uprev, part_u);
+    __syncthreads();
+    if (wave == 0) {
+      if (r >= 1 && prev_valid) {
+        const float u = reduce(part_u);
+        const float z = prev_act ? DT::rnd(prev_a * DT::rnd(u)) : 0.f;
+        const size_t o = (size_t)rb * p.N + prev_row;
+        if (p.z32_out && ((prev_bits >> rj) & 1u)) p.z32_out[o] = z;
+        if (p.zt_out) ((st*)p.zt_out)[o] = DT::fromf(z);
+      }
+      prev_a = a; prev_act = act; prev_valid = valid; prev_bits = bits8; prev_row = row;
+    }
+  };
+
+  CATS_RSTAMP(0);
+  // ---- prologue.  x is fetched and staged before the first weight load goes out, so that its read does not
+  // queue behind the weight requests of the whole machine. -------------------------------------------------------
+  u32x4 g0[kMmaSteps], g1[kMmaSteps], u0[kMmaSteps], u1[kMmaSteps];
+  {
+    // nsteps * 64 operand vectors over kMmaThreads threads = STEPS per thread, all loads in flight together;
+    // batch rows past nb read row 0 and store zeros
+    u32x4 xv[STEPS];
+#pragma unroll
+    for (int k = 0; k < STEPS; k++) {
+      const int i = tid + k * kMmaThreads;
+      const int step = i >> 6, l = i & 63;
+      const int n = l & 15, g = l >> 4, b = n & 7, kh = n >> 3;
+      xv[k] = p.x[(size_t)(b < p.nb ? b : 0) * p.row_vecs + step * 8 + kh * 4 + g];
+    }
+#pragma unroll
+    for (int k = 0; k < STEPS; k++) {
+      const int i = tid + k * kMmaThreads;
+      const int b = i & 7;
+      xs[i] = b < p.nb ? xv[k] : zero4();
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    issue(p.w, 0, g0, false);
+    issue(p.w, 1, g1, false);
+    if (UP) issue(p.w, my_tiles, u1, false);  // defined before the first (unused) up product
+  }
+  __syncthreads();
+  CATS_RSTAMP(1);
+
+  // rounds 0 .. my_tiles: the last one only drains the up sums of the last tile
+  const int last = UP ? my_tiles : my_tiles - 1;
+  for (int r = 0; r <= last; r += 2) {
+    round_body(r, g0, u0, u1);
+    if (r + 1 <= last) round_body(r + 1, g1, u1, u0);
+#ifdef CATS_TIMING
+    if (r < 10) CATS_RSTAMP(2 + (r >> 1));
+#endif
+  }
+  CATS_RSTAMP(7);
+}
+
+}  // namespace cats

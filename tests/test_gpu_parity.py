@@ -276,6 +276,55 @@ def test_config4_small_batch_union(oracle, B):
     assert union_sparsity <= row_sparsity + 1e-6
 
 
+MATRIX_CORE = [
+    # H, I, B, dtype -- 3..8 batch rows in 16-bit types with a row length of 2048 or 4096 take the matrix-core
+    # gate / gate+up kernel (tiles of 8 rows dealt round-robin to one workgroup per CU)
+    (4096, 1003, 3, torch.float16),    # I not a multiple of 8: the last tile has 3 live rows
+    (4096, 520, 5, torch.bfloat16),
+    (2048, 777, 7, torch.float16),
+    (2048, 64, 8, torch.bfloat16),
+    (4096, 8, 4, torch.float16),       # a single tile
+    (4096, 2056, 6, torch.float16),    # 257 tiles: one workgroup gets two, the rest one
+    (2048, 6152, 4, torch.bfloat16),   # 769 tiles: four rounds on the first workgroup, three on the others
+]
+
+
+@pytest.mark.parametrize("H,I,B,dtype", MATRIX_CORE)
+def test_matrix_core_batches(oracle, H, I, B, dtype):
+    m = make_mlp(H, I, B, dtype, seed=H + I + B, corr=0.5)
+    a_abs = oracle.c_gate(m["x"], m["wg"], -1.0)[0].float().abs().flatten()
+    for q in (0.0, 0.5, 0.97):
+        t = -1.0 if q == 0.0 else float(torch.quantile(a_abs, q))
+        check_mlp_case(oracle, m, t, tag=f"matrix-core-q{q}")
+    check_mlp_case(oracle, m, 1e9, tag="matrix-core-all-dead")
+
+
+def test_matrix_core_and_wave_per_row_kernels_agree(oracle):
+    """Same inputs through both gate+up kernels (the tuning knob pins the wave-per-row one): flags may differ only
+    where an activation sits within rounding distance of t, outputs agree to the parity tolerance."""
+    m = make_mlp(4096, 2048, 8, torch.float16, seed=77, corr=0.5)
+    t = calibrate(m["wg"], [0.5])[0]
+    d = dev(m)
+    ws = _ws(8, 4096, 2048)
+    try:
+        capi.set_tuning(-1, 0, 0, 0)
+        y_w, f_w, _ = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
+        a_w, _ = capi.gate_flag(d["x"], d["wg"], t)
+        capi.set_tuning(0, 0, 0, 0)
+        y_m, f_m, _ = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
+        a_m, _ = capi.gate_flag(d["x"], d["wg"], t)
+    finally:
+        capi.set_tuning(0, 0, 0, 0)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(a_m.float().cpu(), a_w.float().cpu(), **A_TOL[torch.float16])
+    flips = (f_w != f_m).cpu()
+    if int(flips.sum()):
+        dist = (a_w.float().cpu().abs() - t).abs()[flips]
+        assert float(dist.max()) <= A_TOL[torch.float16]["atol"] + A_TOL[torch.float16]["rtol"] * abs(t)
+    if int(flips.sum()) == 0:
+        close(y_m.cpu(), y_w.cpu(), torch.float16)
+
+
 def test_reference_recipe_shapes(oracle):
     """The reference's own test recipe: U(-0.5, 0.5) data, (4096 -> 14336), t = 0.2 / 0.3, B = 1 and 2
     (flash_gemv/test/test_fuse_gemv_cmp.py:173-187, 442-524).  Only the gate / mask part is checked at t = 0.2;
