@@ -286,7 +286,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   if (!s_last) return;
   const uint64_t* slabpart = (const uint64_t*)(p.partial + (size_t)slab * p.ngroup * B * kSlabCols);
   constexpr int kPairs = VEC / 2 * kWave;  // 64-bit items per batch row and group
-  constexpr int kInFlight = 16;
+  constexpr int kInFlight = 32;  // with the default 32 groups every partial of an item is requested in one go
   for (int item = tid; item < p.nb * kPairs; item += blockDim.x) {
     const int b = item / kPairs, r = item - b * kPairs;
     const int e = (r >> 6) * 2, l = r & 63;

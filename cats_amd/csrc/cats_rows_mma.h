@@ -1,4 +1,4 @@
-// Fused gate + up pass for batches of 2..8 rows in 16-bit types, on the matrix cores.
+// Gate and fused gate + up pass for batches of 3..8 rows in 16-bit types, on the matrix cores.
 //
 // Why not the wave-per-row kernel: with B batch rows every 16-byte weight vector costs 4 * B v_dot2 and B / 2
 // LDS reads of x per lane.  From B = 4 on, that arithmetic plus the LDS traffic takes as long as the HBM stream
@@ -18,7 +18,7 @@
 //   round r:  MFMA on the gate rows of tile r (loaded two rounds ago) -> per-wave partial sums to LDS;
 //             gate loads of tile r + 2 go out; wave 0 adds the partials in wave order, applies SiLU and the
 //             threshold and publishes the tile's union bits; up loads of tile r go out for the active rows only
-//             (lanes of inactive rows are masked off, so no bytes move for them); MFMA on the up rows of tile
+//             (lanes of inactive rows re-read one cached line, so no HBM bytes move for them); MFMA on the up rows of tile
 //             r - 1 (loaded one round ago) -> partials -> wave 0 writes z = a * up for tile r - 1.
 // So the gate rows of two tiles and the up rows of one are in flight while a fourth tile is being reduced; the
 // only exposed latencies are the first gate load and the last up load.  The two load rings are addressed
