@@ -22,7 +22,7 @@ DTYPE_CODE = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
 SYMBOLS = (
     "cats_version", "cats_status_string", "cats_workspace_bytes", "cats_workspace_init", "cats_gate_flag",
     "cats_gate_compact", "cats_read_count", "cats_up_flag", "cats_down_flag", "cats_gate_up", "cats_mlp",
-    "cats_mlp_rowmajor_down", "cats_set_tuning",
+    "cats_mlp_rowmajor_down", "cats_mlp_norm_residual", "cats_set_tuning",
 )
 
 
@@ -49,6 +49,8 @@ def lib() -> ctypes.CDLL:
         L.cats_gate_up.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp]; L.cats_gate_up.restype = i32
         L.cats_mlp.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_mlp.restype = i32
         L.cats_mlp_rowmajor_down.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_mlp_rowmajor_down.restype = i32
+        L.cats_mlp_norm_residual.argtypes = [vp, vp, f32, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]
+        L.cats_mlp_norm_residual.restype = i32
         L.cats_set_tuning.argtypes = [i32, i32, i32, i32]; L.cats_set_tuning.restype = i32
         _lib = L
     return _lib
@@ -149,6 +151,17 @@ def mlp(x, wgate, wup, wdown_t, threshold, ws: Workspace, y=None, want_flag=Fals
     out = y if y_f32 is None else y_f32
     if want_flag or want_count:
         return out, flag, count
+    return out
+
+
+def mlp_norm_residual(h, norm_weight, eps, wgate, wup, wdown_t, threshold, ws: Workspace, out=None):
+    """out = h + MLP(norm_weight * rms_norm(h)); pass out=h to update the hidden state in place."""
+    B, H, I = _dims(h, wgate)
+    if out is None:
+        out = torch.empty(B, H, dtype=h.dtype, device=h.device)
+    check(lib().cats_mlp_norm_residual(_p(h), _p(norm_weight), float(eps), _p(wgate), _p(wup), _p(wdown_t), _p(out), B, H, I,
+                                       DTYPE_CODE[h.dtype], float(threshold), _p(ws.buf), ws.nbytes, _stream(h)),
+          "cats_mlp_norm_residual")
     return out
 
 

@@ -176,7 +176,7 @@ int do_rows(int mode, int dtype, const RowsArgs& a_in, hipStream_t s) {
 
 // Sparse down over mask words already in the workspace.
 int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_out, int32_t* count_out, int B, int H, int I,
-            int dtype, char* ws, const WsLayout& l, hipStream_t s) {
+            int dtype, char* ws, const WsLayout& l, hipStream_t s, const void* residual = nullptr) {
   DownArgs d;
   memset(&d, 0, sizeof(d));
   d.wd = (const u32x4*)wdown_t;
@@ -184,6 +184,7 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   d.mask = (const uint8_t*)(ws + l.mask);
   d.y32 = y32;
   d.y_out = y_out;
+  d.residual = residual;
   d.partial = (float*)(ws + l.partial);
   d.done = (uint32_t*)(ws + l.counters);
   d.count_out = count_out;
@@ -383,6 +384,31 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
   if (g_tuning.stages == 1) return CATS_OK;
   float* acc = y_f32;
   return do_down(a.z32_out, true, wdown_t, acc, y_out, count_out, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
+}
+
+int cats_mlp_norm_residual(const void* h, const void* norm_weight, float eps, const void* wgate, const void* wup,
+                           const void* wdown_t, void* out, int B, int H, int I, int dtype, float threshold, void* ws,
+                           size_t ws_bytes, void* stream) {
+  int st = check_common(B, H, I, dtype);
+  if (st) return st;
+  if (!h || !norm_weight || !wgate || !wup || !wdown_t || !out) return CATS_ERR_NULL;
+  if (!aligned16(h) || !aligned16(norm_weight) || !aligned16(wgate) || !aligned16(wup) || !aligned16(wdown_t)) return CATS_ERR_ALIGN;
+  // the norm works on the LDS copy of h: same bound as the kernels' own x staging
+  if ((size_t)batch_template(B) * (((size_t)H * elem_size(dtype) + 8191) / 8192 * 8192) > 128 * 1024) return CATS_ERR_SHAPE;
+  WsLayout l;
+  st = check_ws(ws, ws_bytes, H, I, l);
+  if (st) return st;
+  RowsArgs a;
+  fill_rows(a, h, wgate, H, I, B, dtype);
+  a.w2 = (const u32x4*)wup;
+  a.z32_out = (float*)((char*)ws + l.z32);
+  a.mask_out = (uint8_t*)ws + l.mask;
+  a.t = round_through(dtype, threshold);
+  a.norm_w = (const u32x4*)norm_weight;
+  a.norm_eps = eps;
+  st = do_rows(kGateUp, dtype, a, (hipStream_t)stream);
+  if (st) return st;
+  return do_down(a.z32_out, true, wdown_t, nullptr, out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream, h);
 }
 
 int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out, int B, int H,

@@ -108,6 +108,44 @@ struct F32 {
   }
 };
 
+// ---- RMS norm pieces (generic over the traits) ----------------------------------------------------
+// Sum of squares of the VEC elements of one vector, in fp32.
+template <class DT>
+__device__ __forceinline__ float vec_sumsq(u32x4 x, float acc) {
+  return DT::dot(x, x, acc);
+}
+
+// Element-wise  w * round(x * scale)  with both roundings through the storage type: the two steps of an RMS norm
+// layer whose weight multiplies the already down-cast normalised activations.
+template <class DT>
+__device__ __forceinline__ u32x4 vec_norm_apply(u32x4 x, float scale, u32x4 w) {
+  typedef typename DT::st st;
+  constexpr int PER = 4 / sizeof(st);  // elements per dword
+  u32x4 out;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const uint32_t xi = x[i], wi = w[i];  // by value: see as_f16x2
+    uint32_t o = 0;
+#pragma unroll
+    for (int h = 0; h < PER; h++) {
+      st xe, we;
+      if constexpr (PER == 1) {
+        xe = __builtin_bit_cast(st, xi);
+        we = __builtin_bit_cast(st, wi);
+      } else {
+        xe = (st)(xi >> (16 * h));
+        we = (st)(wi >> (16 * h));
+      }
+      const float xn = DT::rnd(DT::tof(xe) * scale);
+      const st r = DT::fromf(DT::tof(we) * xn);
+      if constexpr (PER == 1) o = __builtin_bit_cast(uint32_t, r);
+      else o |= (uint32_t)r << (16 * h);
+    }
+    out[i] = o;
+  }
+  return out;
+}
+
 // ---- wave64 cross-lane helpers ------------------------------------------------------------------
 
 template <int CTRL>

@@ -29,6 +29,7 @@ struct DownArgs {
   const uint8_t* mask;    // ceil(I/8) bytes, bit j = neuron j active for some batch row
   float* y32;             // (nb, H) the caller's fp32 accumulator (atomics), used when y_out == NULL
   void* y_out;            // (nb, H) dtype
+  const void* residual;   // optional (nb, H) dtype, y_out mode: y = residual + round(sum); may alias y_out
   float* partial;         // y_out mode: [nslab][ngroup][B][64*VEC] fp32 slab partials
   uint32_t* done;         // y_out mode: per-slab arrival counters, zero between calls
   int32_t* count_out;     // optional: number of active neurons
@@ -309,6 +310,11 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
     }
     if (col < p.H) {
       st* y = (st*)p.y_out + (size_t)b * p.H + col;
+      if (p.residual) {  // the MLP output is rounded to the storage type first, as a module returning a tensor would
+        const st* res = (const st*)p.residual + (size_t)b * p.H + col;
+        s0 = DT::rnd(s0) + DT::tof(res[0]);
+        s1 = DT::rnd(s1) + DT::tof(res[1]);
+      }
       y[0] = DT::fromf(s0);
       y[1] = DT::fromf(s1);
     }

@@ -39,6 +39,8 @@ struct RowsArgs {
   int row_vecs;          // K / VEC
   float t;               // threshold, already rounded through dtype
   int lds_floor;         // host side only: request at least this much dynamic LDS (caps workgroups per CU); 0 = none
+  const u32x4* norm_w;   // optional (K,) RMS-norm weight: x is replaced by norm_w * round(x * rsqrt(mean(x^2) + norm_eps)) while
+  float norm_eps;        //   it is staged (needs x in LDS); NULL = x is used as given
   int mma;               // host side only: kGateUp with 2..8 batch rows may take the matrix-core kernel
 #ifdef CATS_TIMING
   long long* tbuf;       // [gridDim][8] wall-clock stamps (100 MHz) at phase boundaries, development builds only
@@ -177,6 +179,22 @@ void rows_kernel(RowsArgs p) {
   }
   if (threadIdx.x == 0) s_maskbits = 0u;
   __syncthreads();
+  if (XLDS && p.norm_w) {
+    // RMS norm of each batch row, in place in LDS: one wave adds a row's squares (fixed order), everyone rescales.
+    __shared__ float s_scale[B];
+    for (int b = wave; b < B; b += WAVES) {
+      float ss = 0.f;
+      for (int v = lane; v < p.row_vecs; v += kWave) ss = vec_sumsq<DT>(xs[b * nchv + v], ss);
+      ss = wave_sum(ss);
+      if (lane == 0) s_scale[b] = rsqrtf(ss / (float)p.K + p.norm_eps);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < B * nchv; i += kThreads) {
+      const int b = B == 1 ? 0 : i / nchv, v = i - b * nchv;
+      if (b < p.nb && v < p.row_vecs) xs[i] = vec_norm_apply<DT>(xs[i], s_scale[b], p.norm_w[v]);
+    }
+    __syncthreads();
+  }
   CATS_RSTAMP(1);
 
   float a[R][B];       // gate activation, rounded through dtype

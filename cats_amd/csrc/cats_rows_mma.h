@@ -193,6 +193,26 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
     if (UP) issue(p.w, my_tiles, u1, false);  // defined before the first (unused) up product
   }
   __syncthreads();
+  if (p.norm_w) {
+    // RMS norm in place.  Operand slot i = step * 64 + l holds batch row l % 8, vector step * 8 + (l % 16 / 8) * 4 + l / 16.
+    // Wave b adds the squares of batch row b (kMmaWaves == 8 rows), in a fixed order.
+    __shared__ float s_scale[8];
+    {
+      float ss = 0.f;
+      for (int q = lane; q < nsteps * 8; q += kWave) ss = vec_sumsq<DT>(xs[q * 8 + wave], ss);
+      ss = wave_sum(ss);
+      if (lane == 0) s_scale[wave] = rsqrtf(ss / (float)p.K + p.norm_eps);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < STEPS; k++) {
+      const int i = tid + k * kMmaThreads;
+      const int step = i >> 6, l = i & 63;
+      const int n = l & 15, g = l >> 4, b = n & 7, kh = n >> 3;
+      if (b < p.nb) xs[i] = vec_norm_apply<DT>(xs[i], s_scale[b], p.norm_w[step * 8 + kh * 4 + g]);
+    }
+    __syncthreads();
+  }
   CATS_RSTAMP(1);
 
   // rounds 0 .. my_tiles: the last one only drains the up sums of the last tile

@@ -303,6 +303,27 @@ at::Tensor cats_mlp_op(const at::Tensor& x, const at::Tensor& wgate, const at::T
   return out;
 }
 
+// out = h + MLP(norm_weight * rms_norm(h, eps)): the tail of a decoder layer in two launches.
+at::Tensor cats_mlp_norm_residual_op(const at::Tensor& h, const at::Tensor& norm_weight, const double eps, const at::Tensor& wgate,
+                                     const at::Tensor& wup, const at::Tensor& wdown_t, const double threshold) {
+  check_dev(h, "h");
+  const int B = batch_rows(h, "cats_mlp_norm_residual");
+  const int64_t H = h.size(-1), I = wgate.size(0);
+  check_weight(wgate, h, I, H, "wgate");
+  check_weight(wup, h, I, H, "wup");
+  check_weight(wdown_t, h, I, H, "wdown_t (neuron-major)");
+  TORCH_CHECK(norm_weight.is_cuda() && norm_weight.is_contiguous() && norm_weight.scalar_type() == h.scalar_type() &&
+                  norm_weight.numel() == H && norm_weight.get_device() == h.get_device(),
+              "flash_gemv.cats_mlp_norm_residual: norm_weight must be a contiguous (H,) tensor of h's dtype on h's device");
+  at::Tensor out = at::empty_like(h);
+  hipStream_t s = current_stream(h);
+  Workspace& ws = workspace(h, B, (int)H, (int)I, s);
+  check_status(cats_mlp_norm_residual(h.data_ptr(), norm_weight.data_ptr(), (float)eps, wgate.data_ptr(), wup.data_ptr(), wdown_t.data_ptr(),
+                                      out.data_ptr(), B, (int)H, (int)I, dtype_code(h), (float)threshold, ws.buf.data_ptr(), ws.bytes, s),
+               "cats_mlp_norm_residual");
+  return out;
+}
+
 // Same, also returning the per-row flags (B*I bool) and the number of neurons fetched (int32 scalar tensor).
 std::tuple<at::Tensor, at::Tensor, at::Tensor> cats_mlp_stats_op(const at::Tensor& x, const at::Tensor& wgate, const at::Tensor& wup,
                                                                  const at::Tensor& wdown_t, const double threshold) {
@@ -348,6 +369,7 @@ TORCH_LIBRARY(flash_gemv, m) {
   m.def("cats_up_flag", cats_up_flag_op);
   m.def("cats_down_flag", cats_down_flag_op);
   m.def("cats_mlp", cats_mlp_op);
+  m.def("cats_mlp_norm_residual", cats_mlp_norm_residual_op);
   m.def("cats_mlp_stats", cats_mlp_stats_op);
   m.def("cats_set_tuning", cats_set_tuning_op);
 }

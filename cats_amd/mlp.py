@@ -117,6 +117,18 @@ class CatsMLP(nn.Module):
             self.wdown_t = self.down_proj.weight.detach().t().contiguous()
         return self
 
+    def forward_norm_residual(self, h, norm_weight, eps):
+        """``h + self(norm_weight * rms_norm(h, eps))`` for the decode kernel path (sp_method 3): the post-attention
+        norm is applied while the gate kernel stages h, the residual is added where the down kernel writes."""
+        if not (self.is_profile and self.sp_method == 3 and h.shape[1] == 1):
+            raise RuntimeError("CatsMLP.forward_norm_residual: decode path only (prepare_decode(3), one token per row)")
+        if self.wdown_t is None:
+            raise RuntimeError("CatsMLP: sp_method 3 needs wdown_t (call prepare_decode() once after loading weights)")
+        import flash_gemv
+
+        return flash_gemv.cats_mlp_norm_residual(h, norm_weight, float(eps), self.gate_proj.weight, self.up_proj.weight,
+                                                 self.wdown_t, float(self.dead_threshold))
+
     def _dense_masked(self, x):
         post_act = self.act_fn(self.gate_proj(x))
         dead_neurons = post_act.abs() <= self.dead_threshold

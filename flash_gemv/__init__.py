@@ -91,6 +91,15 @@ def cats_mlp(x, Wgate, Wup, Wdownt, threshold):
     return torch.ops.flash_gemv.cats_mlp(x, Wgate, Wup, Wdownt, threshold)
 
 
+def cats_mlp_norm_residual(h, norm_weight, eps, Wgate, Wup, Wdownt, threshold):
+    """h + CATS_MLP(norm_weight * rms_norm(h, eps)) in the same two launches as cats_mlp.
+
+    The three module calls at the end of the reference's decoder layer (residual = h; h = post_attention_layernorm(h);
+    h = residual + mlp(h), experiments/models/sparse_silu/ugly_utils.py:1036-1057) for decode, batch * seq <= 8.
+    """
+    return torch.ops.flash_gemv.cats_mlp_norm_residual(h, norm_weight, eps, Wgate, Wup, Wdownt, threshold)
+
+
 def cats_mlp_stats(x, Wgate, Wup, Wdownt, threshold):
     """cats_mlp that also returns the (B, I) bool flags and the number of neurons fetched (int32 tensor)."""
     return torch.ops.flash_gemv.cats_mlp_stats(x, Wgate, Wup, Wdownt, threshold)
@@ -121,4 +130,5 @@ __all__ = [
     "mistral_mlp_sparse_direct_index_2d",
     "cats_mlp",
     "cats_mlp_stats",
+    "cats_mlp_norm_residual",
 ]

@@ -122,6 +122,17 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
              uint8_t* flag_out, int32_t* count_out, int B, int H, int I, int dtype, float threshold,
              void* ws, size_t ws_bytes, void* stream);
 
+/* The tail of a decoder layer in two launches:  out = h + MLP(norm_weight * rms_norm(h)).
+ * The RMS norm (fp32 mean of squares, rsqrt(mean + eps), result rounded to dtype, then multiplied by norm_weight in
+ * dtype -- the HF LlamaRMSNorm / MistralRMSNorm order) is applied while the gate+up kernel stages h in LDS; the
+ * residual add happens where the down kernel writes its output (MLP result rounded to dtype first, then added).
+ * h, out (B,H) in dtype; out may alias h.  norm_weight (H) in dtype.  Needs B*H*sizeof(dtype) <= 128 KiB.
+ * Replaces the three module calls  residual = h; h = post_attention_layernorm(h); h = residual + mlp(h)
+ * of the reference's decoder layer (experiments/models/sparse_silu/ugly_utils.py:1036-1057) for batch*seq <= 8. */
+int cats_mlp_norm_residual(const void* h, const void* norm_weight, float eps, const void* wgate, const void* wup,
+                           const void* wdown_t, void* out, int B, int H, int I, int dtype, float threshold,
+                           void* ws, size_t ws_bytes, void* stream);
+
 /* Whole CATS MLP with the HF (H,I) down weight: gate+up, then a dense row-major GEMV over the zero-filled
  * intermediate (all of wdown is read, as in the reference).
  * Replaces flag_gemv_gemv and flag_gemv_gemv_inner{,_fp32,_bf16} (flash_gemv.py:33-43;

@@ -14,7 +14,9 @@ Two independent restatements live here:
   the checker for dtype-exact questions (mask bits on identical gate values).
 
 Parity status: the reference ships no golden vectors for this path; both restatements are pinned by the
-closed forms and brute-force checks in ``tests/test_oracle.py``.
+closed forms and brute-force checks in ``tests/test_oracle.py``.  ``torch_rms_norm`` restates a routine of the
+reference's dependency ``transformers``; it is pinned against the installed library's ``LlamaRMSNorm`` and against
+closed forms there too.
 """
 from __future__ import annotations
 
@@ -88,6 +90,22 @@ def torch_cats_mlp(x, wgate, wup, wdown, threshold):
 def torch_dense_mlp(x, wgate, wup, wdown):
     """Plain SwiGLU MLP (HF LlamaMLP.forward): down(silu(gate(x)) * up(x))."""
     return F.linear(F.silu(F.linear(x, wgate)) * F.linear(x, wup), wdown)
+
+
+def torch_rms_norm(h, weight, eps):
+    """The post-attention norm of the decoder layer the reference patches (ugly_utils.py:1038 calls the HF module).
+    The module lives in the reference's dependency transformers (pinned 4.36.2 in requirements.txt:40), class
+    LlamaRMSNorm / MistralRMSNorm; its published forward is restated here: fp32 mean of squares, rsqrt(mean + eps),
+    cast back to the input dtype, then the weight multiplies in that dtype."""
+    v = h.to(torch.float32)
+    v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    return weight * v.to(h.dtype)
+
+
+def torch_layer_tail(h, norm_weight, eps, wgate, wup, wdown, threshold):
+    """residual = h; h = norm(h); h = residual + mlp(h)  (ugly_utils.py:1036-1057, dense-masked MLP of :895-899)."""
+    y, _, _ = torch_cats_mlp(torch_rms_norm(h, norm_weight, eps), wgate, wup, wdown, threshold)
+    return h + y
 
 
 def torch_flags(x_1, threshold):

@@ -325,6 +325,62 @@ def test_matrix_core_and_wave_per_row_kernels_agree(oracle):
         close(y_m.cpu(), y_w.cpu(), torch.float16)
 
 
+def _gap_threshold(a_abs, q):
+    """A threshold near the q-quantile of |a| that sits in the middle of the widest gap between neighbouring values
+    there, so that a last-bit difference in the normalised input cannot move a neuron across it."""
+    v = torch.sort(a_abs.flatten().float()).values
+    k = int(q * (v.numel() - 1))
+    lo, hi = max(k - 40, 0), min(k + 40, v.numel() - 1)
+    gaps = v[lo + 1:hi + 1] - v[lo:hi]
+    i = int(torch.argmax(gaps)) + lo
+    return float((v[i] + v[i + 1]) / 2)
+
+
+LAYER_TAIL = [
+    # H, I, B, dtype
+    (64, 96, 1, torch.float16), (72, 100, 2, torch.bfloat16), (260, 333, 3, torch.float32),
+    (4096, 1000, 1, torch.float16), (4096, 1003, 5, torch.float16), (2048, 520, 8, torch.bfloat16),
+    (4096, 11008, 1, torch.float16),
+]
+
+
+@pytest.mark.parametrize("H,I,B,dtype", LAYER_TAIL)
+def test_norm_and_residual_folded_into_the_mlp(oracle, H, I, B, dtype):
+    """cats_mlp_norm_residual against  h + MLP(norm(h))  spelled out with the oracle's restatements."""
+    m = make_mlp(H, I, B, dtype, seed=H + 3 * I + B)
+    g = torch.Generator().manual_seed(H + I)
+    h = (m["x"].float() * 2.5 + 0.3).to(dtype)                      # not unit-variance, not zero-mean
+    nw = (1.0 + 0.2 * torch.randn(H, generator=g)).to(dtype)
+    eps = 1e-5
+    x_ref = oracle.torch_rms_norm(h, nw, eps)
+    a_abs = oracle.c_gate(x_ref, m["wg"], -1.0)[0].float().abs()
+    d = dev(dict(h=h, nw=nw, wg=m["wg"], wu=m["wu"], wdt=m["wdt"]))
+    ws = _ws(B, H, I)
+    for q in (0.0, 0.5, 0.9):
+        t = -1.0 if q == 0.0 else _gap_threshold(a_abs, q)
+        print(f"[case] layer-tail dtype={dtype} B={B} H={H} I={I} q={q} t={t}", flush=True)
+        ref = oracle.c_mlp(x_ref, m["wg"], m["wu"], m["wd"], t)
+        want = h + ref["y"].to(dtype)
+        got = capi.mlp_norm_residual(d["h"], d["nw"], eps, d["wg"], d["wu"], d["wdt"], t, ws)
+        # the same thing in two steps on the GPU: torch's norm, the unfused entry point, torch's add
+        two_step = d["h"] + capi.mlp(oracle.torch_rms_norm(d["h"], d["nw"], eps), d["wg"], d["wu"], d["wdt"], t, ws)
+        torch.cuda.synchronize()
+        close(got.cpu(), want, dtype)
+        close(got.cpu(), two_step.cpu(), dtype)
+    # in place: out aliases h
+    h2 = d["h"].clone()
+    capi.mlp_norm_residual(h2, d["nw"], eps, d["wg"], d["wu"], d["wdt"], t, ws, out=h2)
+    torch.cuda.synchronize()
+    assert torch.equal(h2, got)
+
+
+def test_norm_residual_rejects_rows_that_do_not_fit_in_lds():
+    H, I, B = 16384, 64, 8   # 8 x 32 KiB of fp16 activations
+    z = lambda *s: torch.zeros(*s, dtype=torch.float16, device="cuda")
+    with pytest.raises(capi.CatsError, match="shape"):
+        capi.mlp_norm_residual(z(B, H), z(H), 1e-5, z(I, H), z(I, H), z(I, H), 0.1, _ws(B, H, I))
+
+
 def test_reference_recipe_shapes(oracle):
     """The reference's own test recipe: U(-0.5, 0.5) data, (4096 -> 14336), t = 0.2 / 0.3, B = 1 and 2
     (flash_gemv/test/test_fuse_gemv_cmp.py:173-187, 442-524).  Only the gate / mask part is checked at t = 0.2;

@@ -258,3 +258,53 @@ def test_percentile_threshold(oracle):
     assert oracle.percentile_threshold(a, 0.0) == -1.0
     t = oracle.percentile_threshold(a, 0.5)
     assert t == 50.0 and float((a <= t).float().mean()) == 0.5
+
+
+# ---- RMS norm (the decoder layer's post-attention norm, folded into the fused entry point) -----------------------
+
+def test_rms_norm_closed_forms(oracle):
+    # a constant row: mean of squares = c^2, so norm(x) = c / sqrt(c^2 + eps) everywhere
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        h = torch.full((2, 1, 64), 3.0, dtype=dtype)
+        w = torch.full((64,), 0.5, dtype=dtype)
+        got = oracle.torch_rms_norm(h, w, 1e-5)
+        want = 0.5 * 3.0 / (9.0 + 1e-5) ** 0.5
+        assert got.dtype == dtype
+        assert float((got.double() - want).abs().max()) <= want * float(torch.finfo(dtype).eps)
+    # a one-hot row of length n with value v: mean = v^2 / n, norm = sign(v) * sqrt(n) (eps negligible), zeros stay zero
+    h = torch.zeros(1, 1, 256)
+    h[0, 0, 17] = -5.0
+    got = oracle.torch_rms_norm(h, torch.ones(256), 0.0)
+    assert float(got[0, 0, 17]) == pytest.approx(-16.0, rel=1e-6)
+    assert int((got != 0).sum()) == 1
+    # scale invariance: norm(k x) = norm(x) for eps = 0
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(3, 1, 128, generator=g)
+    w = torch.randn(128, generator=g)
+    torch.testing.assert_close(oracle.torch_rms_norm(4.0 * x, w, 0.0), oracle.torch_rms_norm(x, w, 0.0), rtol=1e-6, atol=1e-7)
+
+
+def test_rms_norm_matches_installed_transformers(oracle):
+    """The reference calls the HF module; the installed transformers is a later release than the one the reference
+    pins, the RMS-norm forward is unchanged between them."""
+    mod = pytest.importorskip("transformers.models.llama.modeling_llama")
+    g = torch.Generator().manual_seed(1)
+    for dtype in (torch.float32, torch.float16, torch.bfloat16):
+        n = mod.LlamaRMSNorm(320, eps=1e-5)
+        n.weight.data = torch.randn(320, generator=g).to(dtype)
+        h = (torch.randn(4, 1, 320, generator=g) * 3).to(dtype)
+        assert torch.equal(n(h), oracle.torch_rms_norm(h, n.weight.data, 1e-5))
+
+
+def test_layer_tail_is_residual_plus_mlp_of_norm(oracle):
+    g = torch.Generator().manual_seed(2)
+    H, I = 64, 96
+    h = torch.randn(2, 1, H, generator=g)
+    nw, wg, wu, wd = torch.randn(H, generator=g), torch.randn(I, H, generator=g) * .1, torch.randn(I, H, generator=g) * .1, torch.randn(H, I, generator=g) * .1
+    got = oracle.torch_layer_tail(h, nw, 1e-5, wg, wu, wd, 0.05)
+    x = oracle.torch_rms_norm(h, nw, 1e-5)
+    y, _, _ = oracle.torch_cats_mlp(x, wg, wu, wd, 0.05)
+    assert torch.equal(got, h + y)
+    # with t < 0 nothing is masked: the tail is the plain SwiGLU layer tail
+    dense = h + oracle.torch_dense_mlp(x, wg, wu, wd)
+    torch.testing.assert_close(oracle.torch_layer_tail(h, nw, 1e-5, wg, wu, wd, -1.0), dense)
