@@ -266,7 +266,8 @@ def main():
 
 def other_configs(torch, F, capi, L, steps, warmup):
     """The remaining single-layer configurations: Mistral-7B shape in bf16 with heavy-tailed gate rows (50 / 70 %), and
-    the Llama fp16 layer at batch 2 / 4 / 8 with pairwise-correlated rows (per-row masks, union gathering)."""
+    the Llama fp16 layer at batch 2 / 4 / 8 with pairwise-correlated rows (per-row masks, union gathering), and the
+    Llama-70B-shaped layer at batch 1."""
     import math
 
     dev = torch.device("cuda:0")
@@ -330,6 +331,8 @@ def other_configs(torch, F, capi, L, steps, warmup):
     run("mistral7b_bf16_heavy_tail", 4096, 14336, 1, torch.bfloat16, capi.BF16, [0.5, 0.7], heavy_tail=True)
     for B in (2, 4, 8):
         run(f"llama7b_fp16_batch{B}_corr0.5", 4096, 11008, B, torch.float16, capi.F16, [0.5], corr=0.5)
+    # the larger shape the reference smoke-tests (flash_gemv/test/test_fuse_gemv_cmp.py:662-676): 1.4 GB per weight set
+    run("llama70b_fp16", 8192, 28672, 1, torch.float16, capi.F16, [0.5], nsets=2)
     return res
 
 

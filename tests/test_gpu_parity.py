@@ -381,6 +381,22 @@ def test_norm_residual_rejects_rows_that_do_not_fit_in_lds():
         capi.mlp_norm_residual(z(B, H), z(H), 1e-5, z(I, H), z(I, H), z(I, H), 0.1, _ws(B, H, I))
 
 
+@pytest.mark.parametrize("B", [1, 4])
+def test_llama70b_shape(oracle, B):
+    """8192 -> 28672, the larger shape the reference smoke-tests (flash_gemv/test/test_fuse_gemv_cmp.py:662-676).
+    Rows of 16 KiB: two passes of 8 chunks per row in the wave-per-row kernel, 16 column slabs in the down kernel;
+    batch 4 stays on the wave-per-row kernel (the matrix-core one takes rows of 2048 or 4096 elements)."""
+    m = make_mlp(8192, 28672, B, torch.float16, seed=70, corr=0.5 if B > 1 else 0.0)
+    t = calibrate(m["wg"], [0.5], n_vec=64)[0]
+    check_mlp_case(oracle, m, t, tag=f"llama70b-fp16-B{B}")
+
+
+def test_batch_above_eight_is_an_error_not_a_crash():
+    z = lambda *s: torch.zeros(*s, dtype=torch.float16, device="cuda")
+    with pytest.raises(capi.CatsError, match="batch"):
+        capi.mlp(z(16, 512), z(64, 512), z(64, 512), z(64, 512), 0.1, _ws(8, 512, 64))
+
+
 def test_reference_recipe_shapes(oracle):
     """The reference's own test recipe: U(-0.5, 0.5) data, (4096 -> 14336), t = 0.2 / 0.3, B = 1 and 2
     (flash_gemv/test/test_fuse_gemv_cmp.py:173-187, 442-524).  Only the gate / mask part is checked at t = 0.2;
