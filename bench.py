@@ -253,6 +253,9 @@ def main():
         torch.cuda.empty_cache()
         out["other_configs"] = other_configs(torch, F, capi, L, max(200, args.steps // 4), max(50, args.warmup // 4))
 
+    if not args.no_extra:
+        out["entry_points"] = entry_points(torch, F, capi, max(200, args.steps // 4), max(50, args.warmup // 4))
+
     if args.decode:
         from cats_amd import decoder
 
@@ -333,6 +336,75 @@ def other_configs(torch, F, capi, L, steps, warmup):
         run(f"llama7b_fp16_batch{B}_corr0.5", 4096, 11008, B, torch.float16, capi.F16, [0.5], corr=0.5)
     # the larger shape the reference smoke-tests (flash_gemv/test/test_fuse_gemv_cmp.py:662-676): 1.4 GB per weight set
     run("llama70b_fp16", 8192, 28672, 1, torch.float16, capi.F16, [0.5], nsets=2)
+    return res
+
+
+def entry_points(torch, F, capi, steps, warmup):
+    """Latency of each drop-in entry point alone on the headline layer (Llama shape, fp16, batch 1, 50 % sparsity),
+    with the algorithmic bytes it has to move.  Weight sets rotate as in the headline run."""
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cuda").manual_seed(2)
+    nsets, sz = 6, 2
+    sets = []
+    for _ in range(nsets):
+        wg = (torch.randn(I, H, generator=g, device=dev) * 0.02).half()
+        wu = (torch.randn(I, H, generator=g, device=dev) * 0.02).half()
+        wd = (torch.randn(H, I, generator=g, device=dev) * 0.02).half()
+        sets.append(dict(wg=wg, wu=wu, wd=wd, wdt=wd.t().contiguous()))
+    x = torch.randn(1, H, generator=g, device=dev).half()
+    X = torch.randn(256, H, generator=g, device=dev)
+    act = F.silu(X @ sets[0]["wg"].float().t()).abs().flatten().cpu()
+    t = float(torch.kthvalue(act, int(0.5 * act.numel())).values)
+    ws = capi.Workspace(1, H, I)
+    # per-set inputs of the later stages, produced by the earlier ones
+    for st in sets:
+        st["a"], st["flag"] = capi.gate_flag(x, st["wg"], t)
+        st["z"] = capi.up_flag(x, st["wu"], st["a"], st["flag"])
+    k = sum(int(st["flag"].sum()) for st in sets) / nsets
+    nw = torch.ones(H, dtype=torch.float16, device=dev)
+    # fuse_gemv_cmp: device part only (the reference's op also copies the count to the host, which is a stream sync)
+    vals = torch.empty(I, dtype=torch.float16, device=dev)
+    idx = torch.empty(I, dtype=torch.int64, device=dev)
+    cnt = torch.zeros(1, dtype=torch.int32, device=dev)
+    L = capi.lib()
+    pv = lambda t_: ctypes.c_void_p(t_.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def compact(st):
+        capi.check(L.cats_gate_compact(pv(x), pv(st["wg"]), pv(vals), pv(idx), pv(cnt), H, I, capi.F16, ctypes.c_float(t), pv(ws.buf),
+                                       ws.nbytes, stream), "cats_gate_compact")
+
+    def timed(fn):
+        for i in range(warmup):
+            fn(sets[i % nsets])
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            fn(sets[i % nsets])
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / steps
+
+    full, act_rows = sz * H * I, sz * H * k
+    table = [
+        ("cats_gate_flag", "fuse_gemv_flag / _local / _batch", full, lambda st: capi.gate_flag(x, st["wg"], t)),
+        ("cats_gate_compact", "fuse_gemv_cmp (ordered index list + count, device part)", full, compact),
+        ("cats_up_flag", "fuse_flag_gemv_local, gather_gemv_elemul_flag_3d", act_rows, lambda st: capi.up_flag(x, st["wu"], st["a"], st["flag"])),
+        ("cats_down_flag", "atomic_gemv, gather_transposed_gemv_flag_3d", act_rows, lambda st: capi.down_flag(st["z"], st["wdt"], st["flag"], ws)),
+        ("cats_gate_up", "fuse_gemv_flag_gemv", full + act_rows, lambda st: capi.gate_up(x, st["wg"], st["wu"], t)),
+        ("cats_mlp", "flag_gemv_gemv_atomic, fuse_gemv_flag_gemv_gemv", full + 2 * act_rows, lambda st: capi.mlp(x, st["wg"], st["wu"], st["wdt"], t, ws)),
+        ("cats_mlp_norm_residual", "norm -> mlp -> residual of the decoder layer", full + 2 * act_rows,
+         lambda st: capi.mlp_norm_residual(x, nw, 1e-5, st["wg"], st["wu"], st["wdt"], t, ws)),
+        ("cats_mlp_rowmajor_down", "flag_gemv_gemv, flag_gemv_gemv_inner*", 2 * full + act_rows, lambda st: capi.mlp_rowmajor_down(x, st["wg"], st["wu"], st["wd"], t, ws)),
+    ]
+    res = []
+    for name, replaces, nbytes, fn in table:
+        us = timed(fn)
+        res.append(dict(entry_point=name, replaces=replaces, us=round(us, 2), weight_MB=round(nbytes / 1e6, 1),
+                        GBps=round(nbytes / us * 1e-3, 1), hbm_frac=round(nbytes / us * 1e-3 / HBM_PEAK_GBPS, 4)))
+    del sets
+    torch.cuda.empty_cache()
     return res
 
 

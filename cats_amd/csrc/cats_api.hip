@@ -25,7 +25,7 @@ long long* g_tbuf_down = nullptr;
 #endif
 
 constexpr int kMaxSlabs = 128;
-constexpr size_t kCounterBytes = 1024;  // uint32 words: done[0..127] | arrive 128 | count 192
+constexpr size_t kCounterBytes = 1024 + 64 * 128;  // uint32 words: done[0..127] | arrive 128 | count 192 | 64 arrival sub-counters, one per 128-byte line
 
 __global__ void fill_zero_kernel(u32x4* p, size_t n16) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) p[i] = zero4();
@@ -299,6 +299,7 @@ int cats_gate_compact(const void* x, const void* wgate, void* vals_out, int64_t*
   a.a_out = (char*)ws + l.atmp;
   a.mask_out = (uint8_t*)ws + l.mask;
   a.arrive = (uint32_t*)((char*)ws + l.counters + 512);
+  a.arrive_sub = (uint32_t*)((char*)ws + l.counters + 1024);
   a.idx_out = idx_out;
   a.vals_out = vals_out;
   a.count_out = count_out;

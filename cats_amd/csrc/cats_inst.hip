@@ -1,5 +1,8 @@
 // Kernel instantiations for one dtype.  Compiled three times (-DCATS_DT=F16 / BF16 / F32) so the
 // translation units build in parallel.
+#include <mutex>
+#include <unordered_map>
+
 #include "cats_launch.h"
 #include "cats_rows_mma.h"
 
@@ -10,6 +13,23 @@
 namespace cats {
 
 namespace {
+
+// Kernels that want more than 48 KiB of dynamic LDS have to say so once per process (and again only if a later
+// launch wants more): remembered per kernel so that the launch path makes no runtime call besides the launch.
+hipError_t ensure_dynamic_lds(const void* kern, size_t bytes) {
+  if (bytes <= 48 * 1024) return hipSuccess;
+  static std::mutex mu;
+  static std::unordered_map<uintptr_t, size_t> granted;  // (kernel, device) -> bytes; the attribute is per device
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  const uintptr_t key = (uintptr_t)kern * 64u + (uintptr_t)dev;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = granted.find(key);
+  if (it != granted.end() && it->second >= bytes) return hipSuccess;
+  hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e == hipSuccess) granted[key] = bytes;
+  return e;
+}
 
 constexpr int kR = 2;    // rows per wave per pass
 constexpr int kCB = 8;   // 64-lane chunks whose loads are issued together: 8 x 16 B per lane per row
@@ -26,10 +46,7 @@ hipError_t launch_rows_one(const RowsArgs& a, hipStream_t stream) {
   const int grid = (a.N + rows_per_block - 1) / rows_per_block;
   size_t lds = XLDS ? (size_t)B * ((a.nch + kCB - 1) / kCB * kCB) * kWave * sizeof(u32x4) : 0;
   if ((size_t)a.lds_floor > lds) lds = (size_t)a.lds_floor;
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-  }
+  if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(WAVES * kWave), lds, stream, a);
   return hipGetLastError();
 }
@@ -47,7 +64,7 @@ struct MmaLaunch16 {
     return (steps == 4 || steps == 8) && rows_mma_lds_bytes(a.K) <= 160 * 1024;
   }
   static hipError_t run(const RowsArgs& a, bool up, hipStream_t stream) {
-    static int cus = 0;
+    static int cus = 0;  // one workgroup per CU; every GPU of a node is the same part, so one query serves all
     if (cus == 0) {
       int dev = 0, n = 0;
       if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
@@ -57,8 +74,7 @@ struct MmaLaunch16 {
     auto kern = up ? (s8 ? rows_mma_kernel<DT, 8, true> : rows_mma_kernel<DT, 4, true>)
                    : (s8 ? rows_mma_kernel<DT, 8, false> : rows_mma_kernel<DT, 4, false>);
     const size_t lds = rows_mma_lds_bytes(a.K);
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
+    if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
     const int ntiles = (a.N + kMmaTileRows - 1) / kMmaTileRows;
     hipLaunchKernelGGL(kern, dim3(ntiles < cus ? ntiles : cus), dim3(kMmaThreads), lds, stream, a);
     return hipGetLastError();
@@ -106,10 +122,7 @@ hipError_t launch_down_one(const DownArgs& a, int block, hipStream_t stream) {
   const size_t lds_stream = (size_t)a.chunk * sizeof(int) + (zbytes + 3) / 4 * 4 + (sizeof(typename DT::st) == 2 ? zbytes + 4 * B : 0);
   const size_t lds_fold = (size_t)(nwaves / 2) * B * kWave * DT::VEC * sizeof(float);
   const size_t lds = (lds_stream > lds_fold ? lds_stream : lds_fold) + 64;
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
-  }
+  if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3(a.nslab * a.ngroup), dim3(block), lds, stream, a);
   return hipGetLastError();
 }

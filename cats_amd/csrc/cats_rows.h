@@ -29,6 +29,7 @@ struct RowsArgs {
   void* zt_out;          // kGateUp, kUp, kGemv: (nb, N) dtype, every row written (0 where inactive)
   // compact list, kGate with nb == 1 only
   uint32_t* arrive;      // zeroed counter; the last workgroup to finish builds the list and resets it
+  uint32_t* arrive_sub;  // 64 zeroed counters, 128 bytes apart: first level of the arrival count
   int64_t* idx_out;
   void* vals_out;
   int32_t* count_out;
@@ -249,7 +250,12 @@ void rows_kernel(RowsArgs p) {
 #pragma unroll
           for (int b = 0; b < B; b++)
             if (b < p.nb) {
-              if (MODE == kGate && p.a_out) ((st*)p.a_out)[(size_t)b * p.N + row[r]] = DT::fromf(a[r][b]);
+              if (MODE == kGate && p.a_out) {
+                st* dst = (st*)p.a_out + (size_t)b * p.N + row[r];
+                // read back by another workgroup (the one that builds the list): device-coherent store
+                if (p.idx_out) __hip_atomic_store(dst, DT::fromf(a[r][b]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                else *dst = DT::fromf(a[r][b]);
+              }
               if (p.flag_out) p.flag_out[(size_t)b * p.N + row[r]] = act[r][b] ? 1 : 0;
             }
         }
@@ -289,33 +295,52 @@ void rows_kernel(RowsArgs p) {
       const int nbytes = (p.N + 7) >> 3;
       if (threadIdx.x < kRowsPerBlock / 8) {
         const int byte = blockIdx.x * (kRowsPerBlock / 8) + threadIdx.x;
-        if (byte < nbytes) p.mask_out[byte] = (uint8_t)(s_maskbits >> (8 * threadIdx.x));
+        if (byte < nbytes) {
+          const uint8_t m8 = (uint8_t)(s_maskbits >> (8 * threadIdx.x));
+          if (MODE == kGate && p.idx_out) __hip_atomic_store(&p.mask_out[byte], m8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          else p.mask_out[byte] = m8;
+        }
       }
     }
   }
 
   if (MODE == kGate) {
     if (p.idx_out == nullptr) return;
-    // Last workgroup to arrive turns the mask words into an ascending index list: one neuron per thread,
-    // wave ballot + mbcnt for the rank inside the wave, LDS prefix over the waves, running base per pass.
-    __threadfence();
+    // Last workgroup to arrive turns the mask bytes into an ascending index list: one byte (8 neurons) per thread
+    // and pass, popcount + wave prefix sum + LDS prefix over the waves for the rank, bit expansion for the entries.
+    // No release / acquire fences (at agent scope they write back and invalidate the whole L2): the activations and
+    // mask bytes were stored device-coherently above, each wave waits for its own stores to be acknowledged, the
+    // barrier joins the waves, then the arrival counter is bumped; the last workgroup reads with coherent loads.
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __syncthreads();
     if (threadIdx.x == 0) {
-      const uint32_t prev = __hip_atomic_fetch_add(p.arrive, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-      s_last = prev == gridDim.x - 1;
+      // Two levels: atomics on one address are served one after the other (about 12 ns each), which for a thousand
+      // workgroups would cost more than the gate pass.  Workgroups count into 64 counters on separate lines; the
+      // last one of each counts into the top one.
+      constexpr uint32_t kSub = 64;
+      const uint32_t sub = blockIdx.x % kSub;
+      const uint32_t members = (gridDim.x - sub + kSub - 1) / kSub;
+      uint32_t* sc = p.arrive_sub + sub * 32;
+      bool last = false;
+      if (__hip_atomic_fetch_add(sc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1u) {
+        __hip_atomic_store(sc, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t used = gridDim.x < kSub ? gridDim.x : kSub;
+        last = __hip_atomic_fetch_add(p.arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == used - 1u;
+      }
+      s_last = last;
     }
     __syncthreads();
     if (!s_last) return;
-    __threadfence();
     const st* aall = (const st*)p.a_out;
+    const int nbytes = (p.N + 7) >> 3;
     int base = 0;
-    for (int j0 = 0; j0 < p.N; j0 += kThreads) {
-      const int j = j0 + threadIdx.x;
-      bool bit = false;
-      if (j < p.N) bit = (p.mask_out[j >> 3] >> (j & 7)) & 1;
-      const uint64_t ballot = __ballot(bit);
-      const int rank = ballot_rank(ballot);
-      if (lane == 0) s_wtot[wave] = __popcll(ballot);
+    for (int b0 = 0; b0 < nbytes; b0 += kThreads) {
+      const int byte = b0 + threadIdx.x;
+      uint32_t bits = 0;
+      if (byte < nbytes) bits = __hip_atomic_load(&p.mask_out[byte], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int pc = __popc(bits);
+      const int incl = wave_scan_inclusive(pc, lane);
+      if (lane == kWave - 1) s_wtot[wave] = incl;
       __syncthreads();
       int before = 0, total = 0;
 #pragma unroll
@@ -324,10 +349,22 @@ void rows_kernel(RowsArgs p) {
         if (w < wave) before += c;
         total += c;
       }
-      if (bit) {
-        const int o = base + before + rank;
-        p.idx_out[o] = j;
-        if (p.vals_out) ((st*)p.vals_out)[o] = aall[j];
+      const int o = base + before + incl - pc;
+      // the 8 neurons of the byte, unrolled: all activation loads go out before the first store
+      st v8[8];
+#pragma unroll
+      for (int k = 0; k < 8; k++) {
+        v8[k] = DT::fromf(0.f);
+        if (p.vals_out && ((bits >> k) & 1u))
+          v8[k] = __hip_atomic_load(&aall[byte * 8 + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+#pragma unroll
+      for (int k = 0; k < 8; k++) {
+        if ((bits >> k) & 1u) {
+          const int r = o + __popc(bits & ((1u << k) - 1u));
+          p.idx_out[r] = byte * 8 + k;
+          if (p.vals_out) ((st*)p.vals_out)[r] = v8[k];
+        }
       }
       base += total;
       __syncthreads();
