@@ -186,3 +186,62 @@ def test_decode_loop_graph_replay_matches_eager():
     torch_tokens, _ = model.generate_greedy(prompt, 24, use_graph=False)
     agree = float((torch_tokens == eager).float().mean())
     assert agree >= 0.9, f"only {agree:.2f} of the greedy tokens agree between the HIP and PyTorch CATS paths"
+
+
+def test_graph_replay_of_batched_and_fused_calls():
+    """One HIP graph holding a batch-8 cats_mlp (matrix-core gate+up, batch-8 down) and a cats_mlp_norm_residual
+    call, replayed with fresh inputs between replays and eager work in between: every replay must give what the
+    same calls give eagerly (counters and scratch are left clean by each call, nothing depends on launch order)."""
+    import flash_gemv
+
+    H, I, B = 4096, 1536, 8
+    g = torch.Generator(device="cuda").manual_seed(11)
+    rn = lambda *s: torch.randn(*s, generator=g, device="cuda")
+    wg, wu, wdt = (rn(I, H) * 0.02).half(), (rn(I, H) * 0.02).half(), (rn(I, H) * 0.02).half()
+    nw = (1 + 0.1 * rn(H)).half()
+    x = rn(B, 1, H).half()
+    h = (rn(1, 1, H) * 2).half()
+    t = 0.05
+    # first calls outside the capture: workspaces are allocated and kernel attributes set on first use
+    flash_gemv.cats_mlp(x, wg, wu, wdt, t)
+    flash_gemv.cats_mlp_norm_residual(h, nw, 1e-5, wg, wu, wdt, t)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        flash_gemv.cats_mlp(x, wg, wu, wdt, t)
+        flash_gemv.cats_mlp_norm_residual(h, nw, 1e-5, wg, wu, wdt, t)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            y_g = flash_gemv.cats_mlp(x, wg, wu, wdt, t)
+            h_g = flash_gemv.cats_mlp_norm_residual(h, nw, 1e-5, wg, wu, wdt, t)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        x.copy_(rn(B, 1, H).half())
+        h.copy_((rn(1, 1, H) * 2).half())
+        y_e = flash_gemv.cats_mlp(x, wg, wu, wdt, t)                     # eager, on the default stream
+        h_e = flash_gemv.cats_mlp_norm_residual(h, nw, 1e-5, wg, wu, wdt, t)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_g, y_e), f"replay {rep}: batched MLP differs from the eager call"
+        assert torch.equal(h_g, h_e), f"replay {rep}: fused layer tail differs from the eager call"
+
+
+def test_decode_loop_with_fused_layer_tail():
+    from cats_amd import decoder as dec
+
+    cfg = dec.DecoderConfig(hidden_size=256, intermediate_size=512, num_layers=3, num_heads=4, vocab_size=503, max_len=64)
+    model = dec.LlamaDecoder(cfg, torch.float16, "cuda", seed=0, init_std=0.05).eval()
+    model.calibrate(0.5, n_seq=4, seq_len=16, chunk=4)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    prompt = torch.randint(0, 503, (1, 12), generator=g, device="cuda")
+    model.set_mlp_mode("cats")
+    plain, _ = model.generate_greedy(prompt, 24, use_graph=False)
+    model.set_mlp_mode("cats_fused")
+    fused, _ = model.generate_greedy(prompt, 24, use_graph=False)
+    fused_g, _ = model.generate_greedy(prompt, 24, use_graph=True)
+    assert torch.equal(fused, fused_g)
+    agree = float((plain == fused).float().mean())
+    assert agree >= 0.9, f"only {agree:.2f} of the greedy tokens agree between the fused and the unfused layer tail"
