@@ -189,10 +189,13 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
     }
     __builtin_amdgcn_sched_barrier(0);
     issue(p.w, 0, g0, false);
-    issue(p.w, 1, g1, false);
-    if (UP) issue(p.w, my_tiles, u1, false);  // defined before the first (unused) up product
+#pragma unroll
+    for (int c = 0; c < kMmaSteps; c++) u1[c] = zero4();  // defined before the first (unused) up product
   }
   __syncthreads();
+  // The second gate tile goes out after the barrier: a wave blocks at issue once the CU's miss queue is full, so
+  // everything issued before the barrier delays the moment the staged x becomes usable.
+  issue(p.w, 1, g1, false);
   if (p.norm_w) {
     // RMS norm in place.  Operand slot i = step * 64 + l holds batch row l % 8, vector step * 8 + (l % 16 / 8) * 4 + l / 16.
     // Wave b adds the squares of batch row b (kMmaWaves == 8 rows), in a fixed order.
