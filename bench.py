@@ -57,7 +57,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the Mistral bf16 and batch 2/4/8 configurations")
     ap.add_argument("--no-graph", action="store_true", help="time plain stream launches only")
-    ap.add_argument("--decode", action="store_true", help="also run the 32-layer decode loop (config 5)")
+    ap.add_argument("--decode", action="store_true", help="(default) run the 32-layer decode loop (config 5)")
+    ap.add_argument("--no-decode", action="store_true", help="skip the 32-layer decode loop")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run one 256 MiB device-to-device copy first: a kernel of known traffic for scaling rocprof counters")
     ap.add_argument("--gate-variant", type=int, default=0)
@@ -256,13 +257,20 @@ def main():
     if not args.no_extra:
         out["entry_points"] = entry_points(torch, F, capi, max(200, args.steps // 4), max(50, args.warmup // 4))
 
-    if args.decode:
+    if not args.no_decode:
         from cats_amd import decoder
 
         out["decode"] = decoder.bench_decode(prompt_len=128, gen_len=256, sparsity=0.5)
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, F, thr[0.5] if 0.5 in thr else t50)
+        if not args.no_decode:
+            from cats_amd import decoder
+
+            # the same greedy loop with the dense-masked PyTorch CATS MLP in fp32 on the host cores: 4 of the 32 layers,
+            # 7 timed tokens, per-token time scaled to 32 layers
+            out["cpu_baseline"]["decode"] = decoder.cpu_decode_baseline(num_layers=4, gen_len=8, prompt_len=16, sparsity=0.5,
+                                                                         threads=out["cpu_baseline"]["cores"])
 
     print(json.dumps(out))
 

@@ -270,10 +270,6 @@ def bench_decode(prompt_len=128, gen_len=256, sparsity=0.5, num_layers=32, seed=
         res[f"{mode}_ms_per_token"] = round(secs / (gen_len - 1) * 1e3, 4)
     res["speedup"] = round(res["cats_tok_s"] / res["dense_tok_s"], 3)
     res["speedup_fused"] = round(res["cats_fused_tok_s"] / res["dense_tok_s"], 3)
-    # greedy decoding of a random-init model is chaotic (near-tied logits): the fused path rounds the norm's scale
-    # differently in the last bit, so the two token streams agree for a prefix only
-    same = (toks["cats"] == toks["cats_fused"]).flatten().long()
-    res["fused_tokens_matching_prefix"] = int(same.cumprod(0).sum())
     # achieved union sparsity over the generated tokens is not observable without a sync per layer; report the
     # calibration target and the mean threshold instead
     res["mean_threshold"] = round(sum(thresholds) / len(thresholds), 5)
