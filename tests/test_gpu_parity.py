@@ -119,6 +119,31 @@ def test_small_shapes(oracle, H, I, B, dtype, dist):
         check_mlp_case(oracle, m, t, tag=f"small-{dist}-q{q}")
 
 
+def _random_shapes(n, seed):
+    import random
+
+    rnd = random.Random(seed)
+    out = []
+    for i in range(n):
+        dtype = [torch.float16, torch.bfloat16, torch.float32][i % 3]
+        vec = 4 if dtype == torch.float32 else 8
+        H = vec * rnd.choice([1, 2, 3, 9, 31, 64, 65, 100, 128, 255, 256, 512, 513])   # rows are whole 16-byte vectors
+        I = rnd.choice([1, 2, 7, 8, 9, 63, 64, 65, 127, 200, 343, 344, 345, 1000, 2049])
+        out.append((H, I, rnd.randint(1, 8), dtype))
+    return out
+
+
+@pytest.mark.parametrize("H,I,B,dtype", _random_shapes(24, seed=2024))
+def test_seeded_random_shapes(oracle, H, I, B, dtype):
+    """Odd sizes on purpose: rows of one vector, fewer neurons than a mask byte, ranges that end inside a byte,
+    lists of odd length (the down kernel pairs rows), every batch size."""
+    m = make_mlp(H, I, B, dtype, seed=H * 31 + I * 7 + B)
+    a_abs = oracle.c_gate(m["x"], m["wg"], -1.0)[0].float().abs().flatten()
+    for q in (0.0, 0.4, 0.8):
+        t = -1.0 if q == 0.0 else float(torch.quantile(a_abs, q))
+        check_mlp_case(oracle, m, t, tag=f"random-q{q}")
+
+
 def test_all_dead_and_all_active(oracle):
     m = make_mlp(512, 768, 2, torch.float16, seed=5)
     d = dev(m)
