@@ -55,7 +55,10 @@ def main():
     ap.add_argument("--sparsity", type=float, default=0.5)
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--no-extra", action="store_true", help="skip the Mistral bf16 and batch 2/4/8 configurations")
+    ap.add_argument("--no-extra", action="store_true", help="skip everything but the headline configuration")
+    ap.add_argument("--extra", default="mistral,batch,70b,entry",
+                    help="which of the other measurements to run: mistral (bf16, heavy-tailed), batch (2/4/8), 70b (8192->28672), "
+                         "entry (each drop-in entry point alone)")
     ap.add_argument("--no-graph", action="store_true", help="time plain stream launches only")
     ap.add_argument("--decode", action="store_true", help="(default) run the 32-layer decode loop (config 5)")
     ap.add_argument("--no-decode", action="store_true", help="skip the 32-layer decode loop")
@@ -249,12 +252,13 @@ def main():
         "sweep": sweep,
     }
 
-    if not args.no_extra:
+    extra = set() if args.no_extra else {e.strip() for e in args.extra.split(",") if e.strip()}
+    if extra & {"mistral", "batch", "70b"}:
         del sets
         torch.cuda.empty_cache()
-        out["other_configs"] = other_configs(torch, F, capi, L, max(200, args.steps // 4), max(50, args.warmup // 4))
+        out["other_configs"] = other_configs(torch, F, capi, L, max(200, args.steps // 4), max(50, args.warmup // 4), extra)
 
-    if not args.no_extra:
+    if "entry" in extra:
         out["entry_points"] = entry_points(torch, F, capi, max(200, args.steps // 4), max(50, args.warmup // 4))
 
     if not args.no_decode:
@@ -275,7 +279,7 @@ def main():
     print(json.dumps(out))
 
 
-def other_configs(torch, F, capi, L, steps, warmup):
+def other_configs(torch, F, capi, L, steps, warmup, which):
     """The remaining single-layer configurations: Mistral-7B shape in bf16 with heavy-tailed gate rows (50 / 70 %), and
     the Llama fp16 layer at batch 2 / 4 / 8 with pairwise-correlated rows (per-row masks, union gathering), and the
     Llama-70B-shaped layer at batch 1."""
@@ -339,11 +343,14 @@ def other_configs(torch, F, capi, L, steps, warmup):
         del sets
         torch.cuda.empty_cache()
 
-    run("mistral7b_bf16_heavy_tail", 4096, 14336, 1, torch.bfloat16, capi.BF16, [0.5, 0.7], heavy_tail=True)
-    for B in (2, 4, 8):
-        run(f"llama7b_fp16_batch{B}_corr0.5", 4096, 11008, B, torch.float16, capi.F16, [0.5], corr=0.5)
-    # the larger shape the reference smoke-tests (flash_gemv/test/test_fuse_gemv_cmp.py:662-676): 1.4 GB per weight set
-    run("llama70b_fp16", 8192, 28672, 1, torch.float16, capi.F16, [0.5], nsets=2)
+    if "mistral" in which:
+        run("mistral7b_bf16_heavy_tail", 4096, 14336, 1, torch.bfloat16, capi.BF16, [0.5, 0.7], heavy_tail=True)
+    if "batch" in which:
+        for B in (2, 4, 8):
+            run(f"llama7b_fp16_batch{B}_corr0.5", 4096, 11008, B, torch.float16, capi.F16, [0.5], corr=0.5)
+    if "70b" in which:
+        # the larger shape the reference smoke-tests (flash_gemv/test/test_fuse_gemv_cmp.py:662-676): 1.4 GB per weight set
+        run("llama70b_fp16", 8192, 28672, 1, torch.float16, capi.F16, [0.5], nsets=2)
     return res
 
 
