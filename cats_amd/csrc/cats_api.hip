@@ -25,6 +25,7 @@ long long* g_tbuf_down = nullptr;
 #endif
 
 constexpr int kMaxSlabs = 128;
+constexpr int kKernelBatch = 8;  // rows one launch handles; the entry points take up to CATS_MAX_BATCH rows in passes of this many
 constexpr size_t kCounterBytes = 1024 + 64 * 128;  // uint32 words: done[0..127] | arrive 128 | count 192 | 64 arrival sub-counters, one per 128-byte line
 
 __global__ void fill_zero_kernel(u32x4* p, size_t n16) {
@@ -55,12 +56,12 @@ struct WsLayout {
 
 constexpr int kMaxGroups = 64;  // neuron groups of the sparse down kernel; bounds the partial-sum scratch
 
-// The carving depends on (H, I) only -- every region is sized for CATS_MAX_BATCH rows -- so calls with
+// The carving depends on (H, I) only -- every region is sized for kKernelBatch rows -- so calls with
 // different batch sizes can share one workspace and the region that must stay zero (the counters) never
 // moves onto bytes another call has dirtied.
 WsLayout ws_layout(int H, int I) {
   WsLayout l;
-  const int B = CATS_MAX_BATCH;
+  const int B = kKernelBatch;
   size_t o = 0;
   l.counters = o; o += kCounterBytes;
   l.partial = o;  o += align_up((size_t)kMaxGroups * B * ((size_t)(H + 511) / 512 * 512) * 4, 256);
@@ -141,7 +142,7 @@ int batch_template(int B) { return B <= 1 ? 1 : (B <= 2 ? 2 : (B <= 4 ? 4 : 8));
 
 int check_common(int B, int H, int I, int dtype) {
   if (dtype != CATS_F16 && dtype != CATS_BF16 && dtype != CATS_F32) return CATS_ERR_DTYPE;
-  if (B < 1 || B > CATS_MAX_BATCH) return CATS_ERR_BATCH;
+  if (B < 1 || B > kKernelBatch) return CATS_ERR_BATCH;
   if (H <= 0 || I <= 0) return CATS_ERR_SHAPE;
   if (((size_t)H * elem_size(dtype)) % 16 != 0) return CATS_ERR_ALIGN;
   return CATS_OK;
@@ -225,6 +226,21 @@ int check_ws(const void* ws, size_t ws_bytes, int H, int I, WsLayout& l) {
 
 using namespace cats;
 
+namespace {  // pass helpers of the public entry points
+inline const void* at_cbytes(const void* p, size_t bytes) { return p ? (const char*)p + bytes : nullptr; }
+inline void* at_bytes(void* p, size_t bytes) { return p ? (char*)p + bytes : nullptr; }
+inline size_t esz(int dtype) { return dtype == CATS_F32 ? 4 : 2; }
+template <class F>
+int in_passes(int B, F&& pass) {
+  if (B < 1 || B > CATS_MAX_BATCH) return CATS_ERR_BATCH;
+  for (int b0 = 0; b0 < B; b0 += kKernelBatch) {
+    const int nb = B - b0 < kKernelBatch ? B - b0 : kKernelBatch;
+    if (int st = pass((size_t)b0, nb)) return st;
+  }
+  return CATS_OK;
+}
+}  // namespace
+
 extern "C" {
 
 #ifdef CATS_TIMING
@@ -239,7 +255,7 @@ const char* cats_status_string(int status) {
     case CATS_ERR_DTYPE: return "unsupported dtype (expected 0=fp16, 1=bf16, 2=fp32)";
     case CATS_ERR_SHAPE: return "unsupported shape (H, I must be positive; H <= 128 slabs of 64 x 16 bytes)";
     case CATS_ERR_ALIGN: return "pointer or row pitch not 16-byte aligned";
-    case CATS_ERR_BATCH: return "unsupported batch (1..8 rows)";
+    case CATS_ERR_BATCH: return "unsupported batch (1..16 rows; the active-neuron count is available for 1..8)";
     case CATS_ERR_NULL: return "required pointer is NULL";
     case CATS_ERR_WORKSPACE: return "workspace missing, misaligned (256 bytes) or smaller than cats_workspace_bytes()";
     case CATS_ERR_LAUNCH: return "HIP kernel launch failed";
@@ -271,7 +287,7 @@ int cats_workspace_init(void* ws, size_t ws_bytes, void* stream) {
   return hipGetLastError() == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
 }
 
-int cats_gate_flag(const void* x, const void* wgate, void* a_out, uint8_t* flag_out, int B, int H, int I, int dtype,
+static int gate_flag_pass(const void* x, const void* wgate, void* a_out, uint8_t* flag_out, int B, int H, int I, int dtype,
                    float threshold, void* stream) {
   int st = check_common(B, H, I, dtype);
   if (st) return st;
@@ -315,7 +331,7 @@ int cats_read_count(const int32_t* count_dev, void* stream) {
   return v;
 }
 
-int cats_up_flag(const void* x, const void* wup, const void* a_in, const uint8_t* flag, void* out, int out_is_f32, int B,
+static int up_flag_pass(const void* x, const void* wup, const void* a_in, const uint8_t* flag, void* out, int out_is_f32, int B,
                  int H, int I, int dtype, void* stream) {
   int st = check_common(B, H, I, dtype);
   if (st) return st;
@@ -329,7 +345,7 @@ int cats_up_flag(const void* x, const void* wup, const void* a_in, const uint8_t
   return do_rows(kUp, dtype, a, (hipStream_t)stream);
 }
 
-int cats_down_flag(const void* z, const void* wdown_t, const uint8_t* flag, float* y_f32, void* y_out, int B, int H, int I,
+static int down_flag_pass(const void* z, const void* wdown_t, const uint8_t* flag, float* y_f32, void* y_out, int B, int H, int I,
                    int dtype, void* ws, size_t ws_bytes, void* stream) {
   int st = check_common(B, H, I, dtype);
   if (st) return st;
@@ -346,7 +362,7 @@ int cats_down_flag(const void* z, const void* wdown_t, const uint8_t* flag, floa
   return do_down(z, false, wdown_t, acc, y_out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
 }
 
-int cats_gate_up(const void* x, const void* wgate, const void* wup, void* out, uint8_t* flag_out, int B, int H, int I,
+static int gate_up_pass(const void* x, const void* wgate, const void* wup, void* out, uint8_t* flag_out, int B, int H, int I,
                  int dtype, float threshold, void* stream) {
   int st = check_common(B, H, I, dtype);
   if (st) return st;
@@ -361,7 +377,7 @@ int cats_gate_up(const void* x, const void* wgate, const void* wup, void* out, u
   return do_rows(kGateUp, dtype, a, (hipStream_t)stream);
 }
 
-int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, float* y_f32,
+static int mlp_pass(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, float* y_f32,
              uint8_t* flag_out, int32_t* count_out, int B, int H, int I, int dtype, float threshold, void* ws,
              size_t ws_bytes, void* stream) {
   int st = check_common(B, H, I, dtype);
@@ -387,7 +403,7 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
   return do_down(a.z32_out, true, wdown_t, acc, y_out, count_out, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
 }
 
-int cats_mlp_norm_residual(const void* h, const void* norm_weight, float eps, const void* wgate, const void* wup,
+static int mlp_norm_residual_pass(const void* h, const void* norm_weight, float eps, const void* wgate, const void* wup,
                            const void* wdown_t, void* out, int B, int H, int I, int dtype, float threshold, void* ws,
                            size_t ws_bytes, void* stream) {
   int st = check_common(B, H, I, dtype);
@@ -412,7 +428,7 @@ int cats_mlp_norm_residual(const void* h, const void* norm_weight, float eps, co
   return do_down(a.z32_out, true, wdown_t, nullptr, out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream, h);
 }
 
-int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out, int B, int H,
+static int mlp_rowmajor_down_pass(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out, int B, int H,
                            int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
   int st = check_common(B, H, I, dtype);
   if (st) return st;
@@ -433,6 +449,77 @@ int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, co
   fill_rows(g, (char*)ws + l.zt, wdown, I, H, B, dtype);
   g.zt_out = y_out;
   return do_rows(kGemv, dtype, g, (hipStream_t)stream);
+}
+
+// ---- public entry points: up to CATS_MAX_BATCH rows, in passes of kKernelBatch rows over the weights --------------
+// Decode batches of 1..8 rows are one pass.  Larger ones (the reference's kernels go to 16) re-read the weights per
+// pass; at that size the union of the masks is dense anyway and the path has nothing left to skip.
+
+
+int cats_gate_flag(const void* x, const void* wgate, void* a_out, uint8_t* flag_out, int B, int H, int I, int dtype,
+                   float threshold, void* stream) {
+  const size_t sz = esz(dtype);
+  return in_passes(B, [&](size_t b0, int nb) {
+    return gate_flag_pass(at_cbytes(x, b0 * H * sz), wgate, at_bytes(a_out, b0 * I * sz), (uint8_t*)at_bytes((void*)flag_out, b0 * I), nb, H, I,
+                          dtype, threshold, stream);
+  });
+}
+
+int cats_up_flag(const void* x, const void* wup, const void* a_in, const uint8_t* flag, void* out, int out_is_f32, int B,
+                 int H, int I, int dtype, void* stream) {
+  const size_t sz = esz(dtype);
+  return in_passes(B, [&](size_t b0, int nb) {
+    return up_flag_pass(at_cbytes(x, b0 * H * sz), wup, at_cbytes(a_in, b0 * I * sz), (const uint8_t*)at_cbytes((const void*)flag, b0 * I),
+                        at_bytes(out, b0 * I * (out_is_f32 ? 4 : sz)), out_is_f32, nb, H, I, dtype, stream);
+  });
+}
+
+int cats_down_flag(const void* z, const void* wdown_t, const uint8_t* flag, float* y_f32, void* y_out, int B, int H, int I,
+                   int dtype, void* ws, size_t ws_bytes, void* stream) {
+  const size_t sz = esz(dtype);
+  return in_passes(B, [&](size_t b0, int nb) {
+    return down_flag_pass(at_cbytes(z, b0 * I * sz), wdown_t, (const uint8_t*)at_cbytes((const void*)flag, b0 * I),
+                          (float*)at_bytes((void*)y_f32, b0 * H * 4), at_bytes(y_out, b0 * H * sz), nb, H, I, dtype, ws, ws_bytes, stream);
+  });
+}
+
+int cats_gate_up(const void* x, const void* wgate, const void* wup, void* out, uint8_t* flag_out, int B, int H, int I,
+                 int dtype, float threshold, void* stream) {
+  const size_t sz = esz(dtype);
+  return in_passes(B, [&](size_t b0, int nb) {
+    return gate_up_pass(at_cbytes(x, b0 * H * sz), wgate, wup, at_bytes(out, b0 * I * sz), (uint8_t*)at_bytes((void*)flag_out, b0 * I), nb, H, I,
+                        dtype, threshold, stream);
+  });
+}
+
+int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, float* y_f32,
+             uint8_t* flag_out, int32_t* count_out, int B, int H, int I, int dtype, float threshold, void* ws,
+             size_t ws_bytes, void* stream) {
+  if (count_out && B > kKernelBatch) return CATS_ERR_BATCH;  // the count is that of one pass
+  const size_t sz = esz(dtype);
+  return in_passes(B, [&](size_t b0, int nb) {
+    return mlp_pass(at_cbytes(x, b0 * H * sz), wgate, wup, wdown_t, at_bytes(y_out, b0 * H * sz), (float*)at_bytes((void*)y_f32, b0 * H * 4),
+                    (uint8_t*)at_bytes((void*)flag_out, b0 * I), count_out, nb, H, I, dtype, threshold, ws, ws_bytes, stream);
+  });
+}
+
+int cats_mlp_norm_residual(const void* h, const void* norm_weight, float eps, const void* wgate, const void* wup,
+                           const void* wdown_t, void* out, int B, int H, int I, int dtype, float threshold, void* ws,
+                           size_t ws_bytes, void* stream) {
+  const size_t sz = esz(dtype);
+  return in_passes(B, [&](size_t b0, int nb) {
+    return mlp_norm_residual_pass(at_cbytes(h, b0 * H * sz), norm_weight, eps, wgate, wup, wdown_t, at_bytes(out, b0 * H * sz), nb, H, I, dtype,
+                                  threshold, ws, ws_bytes, stream);
+  });
+}
+
+int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out, int B, int H,
+                           int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
+  const size_t sz = esz(dtype);
+  return in_passes(B, [&](size_t b0, int nb) {
+    return mlp_rowmajor_down_pass(at_cbytes(x, b0 * H * sz), wgate, wup, wdown, at_bytes(y_out, b0 * H * sz), nb, H, I, dtype, threshold, ws,
+                                  ws_bytes, stream);
+  });
 }
 
 }  // extern "C"

@@ -95,7 +95,7 @@ def cats_mlp_norm_residual(h, norm_weight, eps, Wgate, Wup, Wdownt, threshold):
     """h + CATS_MLP(norm_weight * rms_norm(h, eps)) in the same two launches as cats_mlp.
 
     The three module calls at the end of the reference's decoder layer (residual = h; h = post_attention_layernorm(h);
-    h = residual + mlp(h), experiments/models/sparse_silu/ugly_utils.py:1036-1057) for decode, batch * seq <= 8.
+    h = residual + mlp(h), experiments/models/sparse_silu/ugly_utils.py:1036-1057) for decode, batch * seq <= 16.
     """
     return torch.ops.flash_gemv.cats_mlp_norm_residual(h, norm_weight, eps, Wgate, Wup, Wdownt, threshold)
 

@@ -53,7 +53,7 @@ typedef enum {
   CATS_ERR_LAUNCH = 7      /* the HIP runtime refused a launch; hipGetLastError() has details */
 } cats_status_t;
 
-#define CATS_MAX_BATCH 8
+#define CATS_MAX_BATCH 16  /* 1..8 rows are one pass over the weights; 9..16 rows are two (the weights are read per pass) */
 
 /* Library identification / error text.  No reference counterpart (the reference printf()s and exit()s:
  * flash_gemv/csrc/cuda/fuse_gemv_cmp_cuda.cu:25-33,2397-2400). */
@@ -113,7 +113,7 @@ int cats_gate_up(const void* x, const void* wgate, const void* wup, void* out, u
 
 /* Whole CATS MLP with neuron-major down weights: two launches (gate+up, sparse down).
  *   y_out != NULL : (B,H) in dtype;  y_f32 != NULL : fp32 accumulate into the caller's pre-zeroed (B,H).
- * flag_out (B,I) optional.  count_out (device int32, optional) receives the number of neurons fetched
+ * flag_out (B,I) optional.  count_out (device int32, optional, B <= 8 only) receives the number of neurons fetched
  * (union over the batch).
  * Replaces flag_gemv_gemv_atomic, fuse_gemv_gemv_gemv, fuse_gemv_flag_gemv_gemv (flash_gemv.py:12-16,30-31;
  * fuse_gemv_cmp_cuda.cu:786-1244,2196-2253) and the composite gemv_gemv_triton / flag_gemv_gemv_triton
@@ -128,7 +128,7 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
  * residual add happens where the down kernel writes its output (MLP result rounded to dtype first, then added).
  * h, out (B,H) in dtype; out may alias h.  norm_weight (H) in dtype.  Needs B*H*sizeof(dtype) <= 128 KiB.
  * Replaces the three module calls  residual = h; h = post_attention_layernorm(h); h = residual + mlp(h)
- * of the reference's decoder layer (experiments/models/sparse_silu/ugly_utils.py:1036-1057) for batch*seq <= 8. */
+ * of the reference's decoder layer (experiments/models/sparse_silu/ugly_utils.py:1036-1057) for batch*seq <= 16. */
 int cats_mlp_norm_residual(const void* h, const void* norm_weight, float eps, const void* wgate, const void* wup,
                            const void* wdown_t, void* out, int B, int H, int I, int dtype, float threshold,
                            void* ws, size_t ws_bytes, void* stream);

@@ -40,7 +40,7 @@ def test_argument_validation_needs_no_gpu():
     big = 1 << 30
     assert L.cats_gate_flag(p, p, p, p, 1, 64, 96, 9, 0.1, None) == 1            # dtype
     assert L.cats_gate_flag(p, p, p, p, 0, 64, 96, 0, 0.1, None) == 4            # batch
-    assert L.cats_gate_flag(p, p, p, p, 9, 64, 96, 0, 0.1, None) == 4
+    assert L.cats_gate_flag(p, p, p, p, 17, 64, 96, 0, 0.1, None) == 4
     assert L.cats_gate_flag(p, p, p, p, 1, 0, 96, 0, 0.1, None) == 2             # shape
     assert L.cats_gate_flag(p, p, p, p, 1, 60, 96, 0, 0.1, None) == 3            # row pitch 120 B
     assert L.cats_gate_flag(p, p, p, p, 1, 62, 96, 2, 0.1, None) == 3            # fp32 row pitch 248 B

@@ -123,10 +123,12 @@ def test_fuse_gemv_cmp_compact_list(oracle):
 
 
 def test_bad_arguments_raise_not_exit():
-    x = torch.zeros(9, 1, 64, dtype=torch.float16, device="cuda")
+    x = torch.zeros(17, 1, 64, dtype=torch.float16, device="cuda")
     w = torch.zeros(96, 64, dtype=torch.float16, device="cuda")
     with pytest.raises(RuntimeError, match="batch"):
         fg.cats_mlp(x, w, w, w, 0.1)
+    with pytest.raises(RuntimeError, match="batch"):   # the active count is per pass of 8 rows
+        fg.cats_mlp_stats(x[:9], w, w, w, 0.1)
     with pytest.raises(RuntimeError, match="must be"):
         fg.cats_mlp(x[:1], w, w[:, :32].contiguous(), w, 0.1)
     with pytest.raises(RuntimeError, match="dtype"):
