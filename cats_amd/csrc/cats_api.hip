@@ -32,22 +32,6 @@ __global__ void fill_zero_kernel(u32x4* p, size_t n16) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) p[i] = zero4();
 }
 
-// (nb, I) flag bytes -> ceil(I/8) mask bytes, bit j = OR over the batch of flag[b, j].
-__global__ void pack_flags_kernel(const uint8_t* flag, int nb, int I, uint8_t* mask, int nbytes) {
-  const int byte = blockIdx.x * blockDim.x + threadIdx.x;
-  if (byte >= nbytes) return;
-  uint32_t bits = 0;
-  for (int e = 0; e < 8; e++) {
-    const int j = byte * 8 + e;
-    if (j < I) {
-      uint32_t on = 0;
-      for (int b = 0; b < nb; b++) on |= flag[(size_t)b * I + j] != 0 ? 1u : 0u;
-      bits |= on << e;
-    }
-  }
-  mask[byte] = (uint8_t)bits;
-}
-
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct WsLayout {
@@ -177,12 +161,13 @@ int do_rows(int mode, int dtype, const RowsArgs& a_in, hipStream_t s) {
 
 // Sparse down over mask words already in the workspace.
 int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_out, int32_t* count_out, int B, int H, int I,
-            int dtype, char* ws, const WsLayout& l, hipStream_t s, const void* residual = nullptr) {
+            int dtype, char* ws, const WsLayout& l, hipStream_t s, const void* residual = nullptr, const uint8_t* flags = nullptr) {
   DownArgs d;
   memset(&d, 0, sizeof(d));
   d.wd = (const u32x4*)wdown_t;
   d.z = z;
   d.mask = (const uint8_t*)(ws + l.mask);
+  d.flags = flags;
   d.y32 = y32;
   d.y_out = y_out;
   d.residual = residual;
@@ -354,12 +339,9 @@ static int down_flag_pass(const void* z, const void* wdown_t, const uint8_t* fla
   WsLayout l;
   st = check_ws(ws, ws_bytes, H, I, l);
   if (st) return st;
-  const int nbytes = (I + 7) / 8;
-  hipLaunchKernelGGL(pack_flags_kernel, dim3((nbytes + 255) / 256), dim3(256), 0, (hipStream_t)stream, flag, B, I,
-                     (uint8_t*)ws + l.mask, nbytes);
-  if (hipGetLastError() != hipSuccess) return CATS_ERR_LAUNCH;
+  // the down kernel ORs the per-row flag bytes of its range itself: no separate packing launch
   float* acc = y_f32;
-  return do_down(z, false, wdown_t, acc, y_out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
+  return do_down(z, false, wdown_t, acc, y_out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream, nullptr, flag);
 }
 
 static int gate_up_pass(const void* x, const void* wgate, const void* wup, void* out, uint8_t* flag_out, int B, int H, int I,

@@ -27,6 +27,7 @@ struct DownArgs {
   const u32x4* wd;        // (I, H) neuron-major
   const void* z;          // (nb, I) fp32 or dtype
   const uint8_t* mask;    // ceil(I/8) bytes, bit j = neuron j active for some batch row
+  const uint8_t* flags;   // alternative to mask: (nb, I) flag bytes, OR-ed over the batch on the fly; NULL = use mask
   float* y32;             // (nb, H) the caller's fp32 accumulator (atomics), used when y_out == NULL
   void* y_out;            // (nb, H) dtype
   const void* residual;   // optional (nb, H) dtype, y_out mode: y = residual + round(sum); may alias y_out
@@ -119,7 +120,17 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
       const int byte = byte0 + lane;
       uint32_t bits = 0;
       if (byte * 8 < j1) {
-        bits = p.mask[byte];
+        if (p.flags) {  // uniform: per-row flag bytes instead of packed bits
+          for (int e = 0; e < 8; e++) {
+            const int j = byte * 8 + e;
+            uint32_t on = 0;
+            if (j < p.I)
+              for (int b = 0; b < p.nb; b++) on |= p.flags[(size_t)b * p.I + j] != 0 ? 1u : 0u;
+            bits |= on << e;
+          }
+        } else {
+          bits = p.mask[byte];
+        }
         const int rem = j1 - byte * 8;
         if (rem < 8) bits &= (1u << rem) - 1u;
       }
