@@ -247,3 +247,31 @@ def test_decode_loop_with_fused_layer_tail():
     assert torch.equal(fused, fused_g)
     agree = float((plain == fused).float().mean())
     assert agree >= 0.9, f"only {agree:.2f} of the greedy tokens agree between the fused and the unfused layer tail"
+
+
+def test_two_streams_with_their_own_workspaces_do_not_interfere():
+    """Calls on different streams run concurrently on the GPU; each stream has its own workspace (counters, partial
+    sums, mask), so results must equal those of the same calls run one after the other."""
+    import flash_gemv
+
+    H, I = 4096, 2048
+    g = torch.Generator(device="cuda").manual_seed(21)
+    rn = lambda *s: torch.randn(*s, generator=g, device="cuda")
+    wg, wu, wdt = (rn(I, H) * 0.02).half(), (rn(I, H) * 0.02).half(), (rn(I, H) * 0.02).half()
+    xs1 = [rn(1, 1, H).half() for _ in range(6)]
+    xs8 = [rn(8, 1, H).half() for _ in range(6)]
+    t = 0.05
+    want1 = [flash_gemv.cats_mlp(x, wg, wu, wdt, t) for x in xs1]
+    want8 = [flash_gemv.cats_mlp(x, wg, wu, wdt, t) for x in xs8]
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    got1, got8 = [], []
+    for i in range(6):
+        with torch.cuda.stream(s1):
+            got1.append(flash_gemv.cats_mlp(xs1[i], wg, wu, wdt, t))
+        with torch.cuda.stream(s2):
+            got8.append(flash_gemv.cats_mlp(xs8[i], wg, wu, wdt, t))
+    torch.cuda.synchronize()
+    for i in range(6):
+        assert torch.equal(got1[i], want1[i]), f"stream 1, call {i}"
+        assert torch.equal(got8[i], want8[i]), f"stream 2, call {i}"
