@@ -407,6 +407,7 @@ def entry_points(torch, F, capi, steps, warmup):
         ("cats_gate_compact", "fuse_gemv_cmp (ordered index list + count, device part)", full, compact),
         ("cats_up_flag", "fuse_flag_gemv_local, gather_gemv_elemul_flag_3d", act_rows, lambda st: capi.up_flag(x, st["wu"], st["a"], st["flag"])),
         ("cats_down_flag", "atomic_gemv, gather_transposed_gemv_flag_3d", act_rows, lambda st: capi.down_flag(st["z"], st["wdt"], st["flag"], ws)),
+        ("cats_up_down", "gemv_gemv_triton (gate activations given)", 2 * act_rows, lambda st: capi.up_down(x, st["a"], st["wu"], st["wdt"], t, ws)),
         ("cats_gate_up", "fuse_gemv_flag_gemv", full + act_rows, lambda st: capi.gate_up(x, st["wg"], st["wu"], t)),
         ("cats_mlp", "flag_gemv_gemv_atomic, fuse_gemv_flag_gemv_gemv", full + 2 * act_rows, lambda st: capi.mlp(x, st["wg"], st["wu"], st["wdt"], t, ws)),
         ("cats_mlp_norm_residual", "norm -> mlp -> residual of the decoder layer", full + 2 * act_rows,

@@ -385,6 +385,27 @@ static int mlp_pass(const void* x, const void* wgate, const void* wup, const voi
   return do_down(a.z32_out, true, wdown_t, acc, y_out, count_out, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
 }
 
+static int up_down_pass(const void* x, const void* a_in, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,
+                        int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
+  int st = check_common(B, H, I, dtype);
+  if (st) return st;
+  if (!x || !a_in || !wup || !wdown_t || !y_out) return CATS_ERR_NULL;
+  if (!aligned16(x) || !aligned16(wup) || !aligned16(wdown_t)) return CATS_ERR_ALIGN;
+  WsLayout l;
+  st = check_ws(ws, ws_bytes, H, I, l);
+  if (st) return st;
+  RowsArgs a;
+  fill_rows(a, x, wup, H, I, B, dtype);
+  a.a_in = a_in;
+  a.flag_in = nullptr;  // flags = |a| > t, computed where a is read
+  a.t = round_through(dtype, threshold);
+  a.z32_out = (float*)((char*)ws + l.z32);
+  a.mask_out = (uint8_t*)ws + l.mask;
+  st = do_rows(kUp, dtype, a, (hipStream_t)stream);
+  if (st) return st;
+  return do_down(a.z32_out, true, wdown_t, nullptr, y_out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
+}
+
 static int mlp_norm_residual_pass(const void* h, const void* norm_weight, float eps, const void* wgate, const void* wup,
                            const void* wdown_t, void* out, int B, int H, int I, int dtype, float threshold, void* ws,
                            size_t ws_bytes, void* stream) {
@@ -482,6 +503,15 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
   return in_passes(B, [&](size_t b0, int nb) {
     return mlp_pass(at_cbytes(x, b0 * H * sz), wgate, wup, wdown_t, at_bytes(y_out, b0 * H * sz), (float*)at_bytes((void*)y_f32, b0 * H * 4),
                     (uint8_t*)at_bytes((void*)flag_out, b0 * I), count_out, nb, H, I, dtype, threshold, ws, ws_bytes, stream);
+  });
+}
+
+int cats_up_down(const void* x, const void* a, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,
+                 int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
+  const size_t sz = esz(dtype);
+  return in_passes(B, [&](size_t b0, int nb) {
+    return up_down_pass(at_cbytes(x, b0 * H * sz), at_cbytes(a, b0 * I * sz), wup, wdown_t, at_bytes(y_out, b0 * H * sz), nb, H, I, dtype,
+                        threshold, ws, ws_bytes, stream);
   });
 }
 

@@ -21,7 +21,7 @@ struct RowsArgs {
   const u32x4* w;        // (N, K) first weight: wgate (kGate, kGateUp), wup (kUp), W (kGemv)
   const u32x4* w2;       // (N, K) wup for kGateUp
   const void* a_in;      // kUp: (nb, N) gate activations in dtype
-  const uint8_t* flag_in;  // kUp: (nb, N)
+  const uint8_t* flag_in;  // kUp: (nb, N); NULL = derive the flags from a_in:  |a| > t
   void* a_out;           // kGate: (nb, N) dtype, optional
   uint8_t* flag_out;     // kGate, kGateUp: (nb, N), optional
   uint8_t* mask_out;     // kGate, kGateUp: ceil(N/8) bytes, bit j = OR over the batch of flag[b, j]; optional
@@ -209,12 +209,20 @@ void rows_kernel(RowsArgs p) {
       any[r] = false;
 #pragma unroll
       for (int b = 0; b < B; b++) {
-        act[r][b] = on[r] && b < p.nb && p.flag_in[(size_t)b * p.N + row[r]] != 0;
-        a[r][b] = act[r][b] ? DT::tof(ain[(size_t)b * p.N + row[r]]) : 0.f;
+        const bool live = on[r] && b < p.nb;
+        const float av = live ? DT::tof(ain[(size_t)b * p.N + row[r]]) : 0.f;
+        act[r][b] = live && (p.flag_in ? p.flag_in[(size_t)b * p.N + row[r]] != 0 : fabsf(av) > p.t);
+        a[r][b] = act[r][b] ? av : 0.f;
         any[r] = any[r] || act[r][b];
       }
       // flags are per-lane loads of the same address; make the branch below provably wave-uniform
       any[r] = __builtin_amdgcn_readfirstlane((int)any[r]) != 0;
+    }
+    if (p.mask_out && lane == 0) {
+      uint32_t bits = 0u;
+#pragma unroll
+      for (int r = 0; r < R; r++) bits |= (any[r] ? 1u : 0u) << (wave * R + r);
+      if (bits) atomicOr(&s_maskbits, bits);
     }
   } else {
     float g[R][B];
@@ -289,7 +297,7 @@ void rows_kernel(RowsArgs p) {
   }
 
   CATS_RSTAMP(3);
-  if (MODE == kGate || MODE == kGateUp) {
+  if (MODE == kGate || MODE == kGateUp || MODE == kUp) {
     if (p.mask_out) {
       __syncthreads();
       const int nbytes = (p.N + 7) >> 3;

@@ -303,6 +303,24 @@ at::Tensor cats_mlp_op(const at::Tensor& x, const at::Tensor& wgate, const at::T
   return out;
 }
 
+// Sparse up + sparse down given the gate activations x_1 (gemv_gemv_triton of the reference package).
+at::Tensor cats_up_down_op(const at::Tensor& x, const at::Tensor& x_1, const at::Tensor& wup, const at::Tensor& wdown_t, const double threshold) {
+  check_dev(x, "x");
+  check_dev(x_1, "x_1");
+  const int B = batch_rows(x, "cats_up_down");
+  const int64_t H = x.size(-1), I = wup.size(0);
+  check_weight(wup, x, I, H, "wup");
+  check_weight(wdown_t, x, I, H, "wdown_t (neuron-major)");
+  TORCH_CHECK(x_1.scalar_type() == x.scalar_type() && x_1.numel() == (int64_t)B * I, "flash_gemv.cats_up_down: x_1 must hold B*I gate activations of x's dtype");
+  at::Tensor out = at::empty_like(x);
+  hipStream_t s = current_stream(x);
+  Workspace& ws = workspace(x, B, (int)H, (int)I, s);
+  check_status(cats_up_down(x.data_ptr(), x_1.data_ptr(), wup.data_ptr(), wdown_t.data_ptr(), out.data_ptr(), B, (int)H, (int)I, dtype_code(x),
+                            (float)threshold, ws.buf.data_ptr(), ws.bytes, s),
+               "cats_up_down");
+  return out;
+}
+
 // out = h + MLP(norm_weight * rms_norm(h, eps)): the tail of a decoder layer in two launches.
 at::Tensor cats_mlp_norm_residual_op(const at::Tensor& h, const at::Tensor& norm_weight, const double eps, const at::Tensor& wgate,
                                      const at::Tensor& wup, const at::Tensor& wdown_t, const double threshold) {
@@ -370,6 +388,7 @@ TORCH_LIBRARY(flash_gemv, m) {
   m.def("cats_down_flag", cats_down_flag_op);
   m.def("cats_mlp", cats_mlp_op);
   m.def("cats_mlp_norm_residual", cats_mlp_norm_residual_op);
+  m.def("cats_up_down", cats_up_down_op);
   m.def("cats_mlp_stats", cats_mlp_stats_op);
   m.def("cats_set_tuning", cats_set_tuning_op);
 }

@@ -60,10 +60,9 @@ def flag_gemv_gemv_triton(x, Wgate, Wup, Wdownt, threshold):
 
 
 def gemv_gemv_triton(x, x_1, Wup, Wdownt, threshold):
-    """Sparse up / down given the gate activations x_1 (reference __init__.py:45-48)."""
-    flags = torch.abs(x_1) > threshold
-    x = gather_gemv_elemul_flag_3d(x, x_1, Wup, flags)
-    return gather_transposed_gemv_flag_3d(x, Wdownt, flags)
+    """Sparse up / down given the gate activations x_1 (reference __init__.py:45-48).  The flags |x_1| > threshold are
+    derived inside the up kernel (same strict comparison, threshold rounded to x_1's dtype as torch does)."""
+    return torch.ops.flash_gemv.cats_up_down(x, x_1.contiguous(), Wup, Wdownt, threshold)
 
 
 def flag_gemv_gemv_dejavu(x, Wgate, Wup, Wdownt, threshold):

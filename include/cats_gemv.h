@@ -122,6 +122,14 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
              uint8_t* flag_out, int32_t* count_out, int B, int H, int I, int dtype, float threshold,
              void* ws, size_t ws_bytes, void* stream);
 
+/* Sparse up + sparse down given the gate activations:  flags = |a| > t per row,  z = a * (x . wup[j]) for active j,
+ * y = sum over active j of z[j] * wdown_t[j,:].  Two launches; the flags are derived inside the up kernel and
+ * reach the down kernel as mask bytes in the workspace.  a (B,I) in dtype; y_out (B,H) in dtype.
+ * Replaces the composite gemv_gemv_triton(x, x_1, Wup, Wdownt, threshold) (flash_gemv/flash_gemv/__init__.py:45-48),
+ * the call the reference's sp_method 2 branch makes (experiments/models/sparse_silu/ugly_utils.py:887-894). */
+int cats_up_down(const void* x, const void* a, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,
+                 int dtype, float threshold, void* ws, size_t ws_bytes, void* stream);
+
 /* The tail of a decoder layer in two launches:  out = h + MLP(norm_weight * rms_norm(h)).
  * The RMS norm (fp32 mean of squares, rsqrt(mean + eps), result rounded to dtype, then multiplied by norm_weight in
  * dtype -- the HF LlamaRMSNorm / MistralRMSNorm order) is applied while the gate+up kernel stages h in LDS; the

@@ -209,6 +209,28 @@ def test_batch_rows_are_independent(oracle):
         torch.testing.assert_close(y1[0].float(), yb[b].float(), **TOL[torch.float16])
 
 
+@pytest.mark.parametrize("H,I,B,dtype", [(4096, 1000, 1, torch.float16), (520, 333, 3, torch.bfloat16), (260, 96, 8, torch.float32),
+                                         (4096, 11008, 1, torch.float16), (512, 200, 12, torch.float16)])
+def test_up_down_given_the_gate_activations(oracle, H, I, B, dtype):
+    """cats_up_down (the reference's gemv_gemv_triton): the caller supplies a = act(gate(x)); flags = |a| > t are derived
+    on the device and must be the ones torch derives; output against the oracle on those activations and flags."""
+    m = make_mlp(H, I, B, dtype, seed=3 * H + I + B)
+    a = oracle.c_gate(m["x"], m["wg"], -1.0)[0]                       # (B, I) in dtype
+    t = float(torch.quantile(a.float().abs().flatten(), 0.5))
+    flag = torch.abs(a) > t
+    d = dev(m)
+    ws = _ws(B, H, I)
+    y = capi.up_down(d["x"], a.cuda(), d["wu"], d["wdt"], t, ws)
+    torch.cuda.synchronize()
+    ref = oracle.c_mlp(m["x"], m["wg"], m["wu"], m["wd"], t, a_in=a, flag_in=flag)
+    close(y.cpu(), ref["y"], dtype)
+    # and the two-call spelling gives the same bits
+    z = capi.up_flag(d["x"], d["wu"], a.cuda(), flag.cuda())
+    y2 = capi.down_flag(z, d["wdt"], flag.cuda(), ws)
+    torch.cuda.synchronize()
+    close(y.cpu(), y2.cpu(), dtype)
+
+
 def test_gate_compact_list(oracle):
     for (H, I, dtype) in ((64, 96, torch.float16), (512, 1000, torch.bfloat16), (4096, 2048, torch.float16), (256, 300, torch.float32)):
         m = make_mlp(H, I, 1, dtype, seed=31)
