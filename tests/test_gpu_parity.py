@@ -9,7 +9,7 @@ import math
 import pytest
 import torch
 
-from tests.util import A_TOL, TOL, calibrate, dev, make_mlp
+from tests.util import A_TOL, TOL, calibrate, dev, load_golden, make_mlp
 
 pytestmark = pytest.mark.gpu
 
@@ -143,6 +143,27 @@ def test_seeded_random_shapes(oracle, H, I, B, dtype):
     for q in (0.0, 0.4, 0.8):
         t = -1.0 if q == 0.0 else float(torch.quantile(a_abs, q))
         check_mlp_case(oracle, m, t, tag=f"random-q{q}")
+
+
+def test_frozen_vectors():
+    """The committed vectors (tests/golden): flags bit-exact wherever the activation is not within rounding distance of
+    the threshold, activations and outputs to the parity tolerance."""
+    for name, c in load_golden().items():
+        dtype = c["dtype"]
+        B, H = c["x"].shape
+        I = c["wg"].shape[0]
+        d = {k: c[k].cuda() for k in ("x", "wg", "wu", "wdt")}
+        a, flag = capi.gate_flag(d["x"], d["wg"], c["t"])
+        y = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], c["t"], _ws(B, H, I))
+        torch.cuda.synchronize()
+        a, flag, y = a.cpu(), flag.cpu(), y.cpu()
+        torch.testing.assert_close(a.float(), c["a"].float(), **A_TOL[dtype])
+        flips = flag != c["flag"]
+        if int(flips.sum()):
+            band = A_TOL[dtype]["atol"] + A_TOL[dtype]["rtol"] * abs(c["t"])
+            assert float((c["a"].float().abs() - c["t"]).abs()[flips].max()) <= band, name
+        else:
+            close(y, c["y"], dtype)
 
 
 def test_all_dead_and_all_active(oracle):

@@ -13,7 +13,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from tests.util import make_mlp
+from tests.util import load_golden, make_mlp
 
 DTYPES = [torch.float16, torch.bfloat16, torch.float32]
 
@@ -308,3 +308,23 @@ def test_layer_tail_is_residual_plus_mlp_of_norm(oracle):
     # with t < 0 nothing is masked: the tail is the plain SwiGLU layer tail
     dense = h + oracle.torch_dense_mlp(x, wg, wu, wd)
     torch.testing.assert_close(oracle.torch_layer_tail(h, nw, 1e-5, wg, wu, wd, -1.0), dense)
+
+
+# ---- frozen vectors --------------------------------------------------------------------------------------------
+
+def test_oracle_reproduces_the_frozen_vectors_bit_for_bit(oracle):
+    """tests/golden/cats_mlp_small.npz was written by this oracle (see make_fixtures.py there for why it is not a
+    reference output); any change of its rounding points or accumulation shows up here."""
+    cases = load_golden()
+    assert set(cases) == {"f16_b1", "f16_b3", "bf16_b2", "f32_b2"}
+    for name, c in cases.items():
+        ref = oracle.c_mlp(c["x"], c["wg"], c["wu"], c["wd"], c["t"])
+        assert torch.equal(ref["flag"], c["flag"]), name
+        assert torch.equal(ref["a"].view(torch.int16 if c["dtype"] != torch.float32 else torch.int32),
+                           c["a"].view(torch.int16 if c["dtype"] != torch.float32 else torch.int32)), name
+        assert torch.equal(ref["y"].view(torch.int16 if c["dtype"] != torch.float32 else torch.int32),
+                           c["y"].view(torch.int16 if c["dtype"] != torch.float32 else torch.int32)), name
+        # and the literal PyTorch formula agrees with the frozen output to the parity tolerance
+        y_t, _, dead = oracle.torch_cats_mlp(c["x"].float(), c["wg"].float(), c["wu"].float(), c["wd"].float(), c["t"])
+        if torch.equal(~dead, c["flag"]):
+            torch.testing.assert_close(y_t, c["y"].float(), rtol=1e-2, atol=2e-3 * max(1.0, float(c["y"].float().abs().max())))

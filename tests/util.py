@@ -67,3 +67,33 @@ def calibrate(wg, sparsities, n_vec=256, seed=1234):
 
 def dev(d, device="cuda"):
     return {k: v.to(device) for k, v in d.items()}
+
+
+def load_golden():
+    """tests/golden/cats_mlp_small.npz as {case: dict of CPU tensors + t}.  The file holds storage bits (npz has no
+    bfloat16); the dtype is in the case name."""
+    from pathlib import Path
+
+    import numpy as np
+
+    z = np.load(Path(__file__).resolve().parent / "golden" / "cats_mlp_small.npz")
+    cases = {}
+    for key in z.files:
+        name, field = key.split("/")
+        cases.setdefault(name, {})[field] = z[key]
+    out = {}
+    for name, c in cases.items():
+        dtype = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}[name.split("_")[0]]
+
+        def dec(arr, dtype=dtype):
+            if dtype == torch.float32:
+                return torch.from_numpy(arr.astype("int64").astype("uint32").view("int32").copy()).view(torch.float32)
+            return torch.from_numpy(arr.view("int16").copy()).view(dtype)
+
+        d = {k: dec(c[k]) for k in ("x", "wg", "wu", "wd", "a", "y")}
+        d["flag"] = torch.from_numpy(c["flag"].copy()).bool()
+        d["t"] = float(c["t"])
+        d["wdt"] = d["wd"].t().contiguous()
+        d["dtype"] = dtype
+        out[name] = d
+    return out
