@@ -212,45 +212,73 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   }
 
   CATS_STAMP(2);
-  // ---- 3. fold the waves pairwise through LDS (upper half writes, lower half adds), log2(nwaves) rounds ------
-  __syncthreads();  // the list and z are dead from here on; their LDS is reused
-  for (int half = nwaves >> 1; half >= 1; half >>= 1) {
-    if (wave >= half && wave < 2 * half) {
-      float* dst = s_red + (size_t)(wave - half) * B * kSlabCols;
-#pragma unroll
-      for (int b = 0; b < B; b++)
-#pragma unroll
-        for (int e = 0; e < VEC; e++) dst[(b * VEC + e) * kWave + lane] = acc[b][e];
-    }
-    __syncthreads();
-    if (wave < half) {
-      const float* src = s_red + (size_t)wave * B * kSlabCols;
-#pragma unroll
-      for (int b = 0; b < B; b++)
-#pragma unroll
-        for (int e = 0; e < VEC; e++) acc[b][e] += src[(b * VEC + e) * kWave + lane];
-    }
-    __syncthreads();
-  }
-
-  // wave 0 holds the slab partial: lane l, element e is column (slab*64 + l) * VEC + e
+  // ---- 3. fold the waves through LDS -----------------------------------------------------------------------
+  // One or two batch rows: every wave writes its sums, one barrier, one thread per column adds the waves in wave
+  // order and stores the slab partial.  More batch rows would not fit in LDS that way: pairwise rounds instead
+  // (upper half writes, lower half adds), after which wave 0 holds the partial.
+  // Partial layout (both ways): float (b, pair p, lane l, k) at b*kSlabCols + p*128 + l*2 + k  is column
+  // (slab*64 + l) * VEC + 2p + k.
   float* mypart = p.partial + ((size_t)slab * p.ngroup + group) * B * kSlabCols;
-  if (wave == 0) {
+  __syncthreads();  // the list and z are dead from here on; their LDS is reused
+  if constexpr (B <= 2) {
+    {
+      float* dst = s_red + (size_t)wave * B * kSlabCols + lane * 2;
 #pragma unroll
-    for (int b = 0; b < B; b++) {
-      if (b < p.nb) {  // uniform
-        if (p.y_out) {
+      for (int b = 0; b < B; b++)
 #pragma unroll
-          for (int e = 0; e < VEC; e += 2) {
-            const uint64_t two = (uint64_t)__float_as_uint(acc[b][e]) | ((uint64_t)__float_as_uint(acc[b][e + 1]) << 32);
-            __hip_atomic_store((uint64_t*)&mypart[((b * VEC + e) >> 1) * (2 * kWave) + 2 * lane], two, __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-          }
-        } else {
+        for (int e = 0; e < VEC; e += 2) {
+          float2 v2 = {acc[b][e], acc[b][e + 1]};
+          *(float2*)(dst + b * kSlabCols + (e >> 1) * (2 * kWave)) = v2;
+        }
+    }
+    __syncthreads();
+    for (int f = tid; f < p.nb * kSlabCols; f += blockDim.x) {
+      float s = 0.f;
+      for (int w = 0; w < nwaves; w++) s += s_red[(size_t)w * B * kSlabCols + f];
+      if (p.y_out) {
+        __hip_atomic_store(&mypart[f], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+        const int b = f / kSlabCols, c = f - b * kSlabCols;
+        const int col = (slab * kWave + ((c & (2 * kWave - 1)) >> 1)) * VEC + (c / (2 * kWave)) * 2 + (c & 1);
+        if (col < p.H && n > 0) unsafeAtomicAdd(&p.y32[(size_t)b * p.H + col], s);
+      }
+    }
+  } else {
+    for (int half = nwaves >> 1; half >= 1; half >>= 1) {
+      if (wave >= half && wave < 2 * half) {
+        float* dst = s_red + (size_t)(wave - half) * B * kSlabCols;
 #pragma unroll
-          for (int e = 0; e < VEC; e++) {
-            const int col = (slab * kWave + lane) * VEC + e;
-            if (col < p.H && n > 0) unsafeAtomicAdd(&p.y32[(size_t)b * p.H + col], acc[b][e]);
+        for (int b = 0; b < B; b++)
+#pragma unroll
+          for (int e = 0; e < VEC; e++) dst[(b * VEC + e) * kWave + lane] = acc[b][e];
+      }
+      __syncthreads();
+      if (wave < half) {
+        const float* src = s_red + (size_t)wave * B * kSlabCols;
+#pragma unroll
+        for (int b = 0; b < B; b++)
+#pragma unroll
+          for (int e = 0; e < VEC; e++) acc[b][e] += src[(b * VEC + e) * kWave + lane];
+      }
+      __syncthreads();
+    }
+    if (wave == 0) {
+#pragma unroll
+      for (int b = 0; b < B; b++) {
+        if (b < p.nb) {  // uniform
+          if (p.y_out) {
+#pragma unroll
+            for (int e = 0; e < VEC; e += 2) {
+              const uint64_t two = (uint64_t)__float_as_uint(acc[b][e]) | ((uint64_t)__float_as_uint(acc[b][e + 1]) << 32);
+              __hip_atomic_store((uint64_t*)&mypart[b * kSlabCols + (e >> 1) * (2 * kWave) + 2 * lane], two, __ATOMIC_RELAXED,
+                                 __HIP_MEMORY_SCOPE_AGENT);
+            }
+          } else {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+              const int col = (slab * kWave + lane) * VEC + e;
+              if (col < p.H && n > 0) unsafeAtomicAdd(&p.y32[(size_t)b * p.H + col], acc[b][e]);
+            }
           }
         }
       }
@@ -281,17 +309,16 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   // ---- 4. last workgroup of the slab adds the partials in group order and writes y ---------------------------
   // Ordering without a release / acquire fence pair (at agent scope those write back and invalidate the whole
   // L2 of the XCD, which costs far more than this kernel): partials are written and read with agent-scope
-  // atomic stores / loads, which are coherent across the device by themselves.  The storing wave waits until
-  // its stores have been acknowledged (s_waitcnt vmcnt(0)) and only then bumps the slab counter -- so when a
+  // atomic stores / loads, which are coherent across the device by themselves.  Every wave waits until its own
+  // stores have been acknowledged (s_waitcnt vmcnt(0)), the barrier joins them, and only then is the slab counter bumped -- so when a
   // workgroup reads "I am last" every partial of the slab is in place, and the loads below, issued after
   // that read, see them.
-  if (wave == 0) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt / lgkmcnt untouched
-    CATS_STAMP(4);
-    if (lane == 0) {
-      const uint32_t prev = __hip_atomic_fetch_add(&p.done[slab], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      s_last = prev == (uint32_t)p.ngroup - 1u;
-    }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt / lgkmcnt untouched: this wave's partial stores are acknowledged
+  __syncthreads();                     // ... and so are everybody else's
+  CATS_STAMP(4);
+  if (tid == 0) {
+    const uint32_t prev = __hip_atomic_fetch_add(&p.done[slab], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = prev == (uint32_t)p.ngroup - 1u;
   }
   __syncthreads();
   CATS_STAMP(5);
