@@ -213,14 +213,14 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
 
   CATS_STAMP(2);
   // ---- 3. fold the waves through LDS -----------------------------------------------------------------------
-  // One or two batch rows: every wave writes its sums, one barrier, one thread per column adds the waves in wave
+  // Up to four batch rows (16 waves x 4 x 2 KiB = 128 KiB of LDS): every wave writes its sums, one barrier, one thread per column adds the waves in wave
   // order and stores the slab partial.  More batch rows would not fit in LDS that way: pairwise rounds instead
   // (upper half writes, lower half adds), after which wave 0 holds the partial.
   // Partial layout (both ways): float (b, pair p, lane l, k) at b*kSlabCols + p*128 + l*2 + k  is column
   // (slab*64 + l) * VEC + 2p + k.
   float* mypart = p.partial + ((size_t)slab * p.ngroup + group) * B * kSlabCols;
   __syncthreads();  // the list and z are dead from here on; their LDS is reused
-  if constexpr (B <= 2) {
+  if constexpr (B <= 4) {
     {
       float* dst = s_red + (size_t)wave * B * kSlabCols + lane * 2;
 #pragma unroll
