@@ -1,8 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the CATS sparse-MLP decode path on one MI355X.
 
-A "step" is one CATS MLP call (gate GEMV + SiLU + threshold + sparse up, then sparse down) on a
-Llama-2-7B-shaped layer (4096 -> 11008), fp16, batch 1, threshold at the 50th percentile of |SiLU(gate)| --
+A "step" is one CATS MLP call (gate GEMV + SiLU + threshold + sparse up + sparse down, then the reduction over
+the workgroups' partial sums) on a Llama-2-7B-shaped layer (4096 -> 11008), fp16, batch 1, threshold at the 50th percentile of |SiLU(gate)| --
 the configuration the headline metric is quoted on.  Inputs are resident in HBM before the timed region.
 Steps rotate over several independent weight sets whose total size exceeds the 256 MB memory-side cache,
 so every step streams its weights from HBM.
@@ -26,9 +26,10 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
-# HBM bytes per launch of the gate+up kernel at 50 % sparsity, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a
-# 256 MiB copy (the committed counter summary under profiles/): 132631 KiB read + 55 KiB written.
-MEASURED_HBM_BYTES_GATE_UP = int((132631 + 55) * 1024)
+# HBM bytes per launch of the dominant kernel at 50 % sparsity, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a copy of
+# known size.  The record names the kernel sources it was measured on (a hash); if they have changed since, the figure
+# is stale and `roofline.traffic` is reported as null.
+TRAFFIC_RECORD = ROOT / "profiles" / "cats_mlp_llama7b_fp16_b1_s50_hbm_traffic.json"
 H, I = 4096, 11008
 SPARSITIES = [0.0, 0.3, 0.5, 0.7, 0.9]
 
@@ -39,11 +40,37 @@ def touched_bytes(sz, B, k):
     return sz * H * I + 2 * sz * H * k + sz * B * (2 * H + I) + 4 * k + 4
 
 
-def stage_bytes(sz, B, k):
-    """Algorithmic bytes per launch of the two kernels: (gate+up, down)."""
-    gate_up = sz * H * I + sz * H * k + sz * B * H + I // 8 + 4 * B * k
-    down = sz * H * k + 4 * B * k + I // 8 + sz * B * H
-    return gate_up, down
+def stage_bytes(sz, B, k, grid=256):
+    """Algorithmic bytes per launch of the two kernels of the single-pass path: (streaming kernel, reduction).
+    Streaming: all of W_gate, k rows each of W_up and W_down^T, x, and the fp32 partial sums it leaves per workgroup;
+    reduction: those partial sums and y."""
+    partials = grid * B * H * 4
+    stream = sz * H * I + 2 * sz * H * k + sz * B * H + partials
+    reduce = partials + sz * B * H
+    return stream, reduce
+
+
+def csrc_hash():
+    """sha256 over the kernel sources, in name order: ties a committed counter reading to the code it was taken on."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for f in sorted((ROOT / "cats_amd" / "csrc").iterdir()):
+        if f.suffix in (".h", ".hip", ".cpp"):
+            h.update(f.name.encode())
+            h.update(f.read_bytes())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic():
+    """(bytes or None, note) from the committed counter record, None if it was taken on other kernel sources."""
+    try:
+        rec = json.loads(TRAFFIC_RECORD.read_text())
+    except (OSError, ValueError):
+        return None, f"no counter record at {TRAFFIC_RECORD.name}"
+    if rec.get("csrc_hash") != csrc_hash():
+        return None, f"counter record {TRAFFIC_RECORD.name} was taken on other kernel sources ({rec.get('csrc_hash')} != {csrc_hash()})"
+    return int(rec["fetch_bytes"] + rec["write_bytes"]), f"{TRAFFIC_RECORD.name}: {rec.get('kernel')}"
 
 
 def main():
@@ -64,10 +91,15 @@ def main():
     ap.add_argument("--no-decode", action="store_true", help="skip the 32-layer decode loop")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run one 256 MiB device-to-device copy first: a kernel of known traffic for scaling rocprof counters")
+    ap.add_argument("--print-csrc-hash", action="store_true", help="print the hash of the kernel sources (for a new counter record) and exit")
+    ap.add_argument("--path", type=int, default=0, help="1 = keep the call on the separate gate+up and sparse-down kernels")
     ap.add_argument("--gate-variant", type=int, default=0)
     ap.add_argument("--down-groups", type=int, default=0)
     ap.add_argument("--down-block", type=int, default=0)
     args = ap.parse_args()
+    if args.print_csrc_hash:
+        print(csrc_hash())
+        return
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the path needs no collective); --gpus must be 1", file=sys.stderr)
         sys.exit(2)
@@ -82,7 +114,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     dtype, sz, B = torch.float16, 2, 1
-    capi.set_tuning(args.gate_variant, args.down_groups, args.down_block, 0)
+    capi.set_tuning(args.gate_variant, args.down_groups, args.down_block, args.path)
 
     if args.copy_calibration:
         src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
@@ -140,14 +172,41 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e3 / steps  # us per step
 
-    def time_cats(t, steps, warmup, stages=0):
-        capi.set_tuning(args.gate_variant, args.down_groups, args.down_block, stages)
+    def time_cats(t, steps, warmup, stage=0):
+        """stage 0: the whole call; 1 / 2: one of its two launches alone, back to back (cats_mlp_stage)."""
         prepared = [mlp_args(st, t) for st in sets]
         n = len(prepared)
-        fn = L.cats_mlp
-        us = time_region(lambda i: fn(*prepared[i % n]), steps, warmup)
-        capi.set_tuning(args.gate_variant, args.down_groups, args.down_block, 0)
+        if stage:
+            stage_args = [(stage,) + a[:5] + a[8:] for a in prepared]  # no y_f32 / flag_out / count_out
+            fn = lambda i: L.cats_mlp_stage(*stage_args[i % n])
+        else:
+            fn = lambda i: L.cats_mlp(*prepared[i % n])
+        capi.check(fn(0), "cats_mlp (first timed-configuration call)")
+        us = time_region(fn, steps, warmup)
+        capi.check(fn(0), "cats_mlp (after the timed region)")
         return us
+
+    def per_rep_stats(t, reps):
+        """Every call between its own pair of events (the reference's bench/utils.py:44-58 times one call per rep and
+        reports the geometric mean; its cache flush is the weight-set rotation here)."""
+        prepared = [mlp_args(st, t) for st in sets]
+        n = len(prepared)
+        for i in range(n * 4):
+            L.cats_mlp(*prepared[i % n])
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        torch.cuda.synchronize()
+        for i, (e0, e1) in enumerate(ev):
+            e0.record()
+            L.cats_mlp(*prepared[i % n])
+            e1.record()
+        torch.cuda.synchronize()
+        us = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in ev)
+        import math
+
+        gmean = math.exp(sum(math.log(max(u, 1e-3)) for u in us) / len(us))
+        return dict(reps=reps, median_us=round(us[len(us) // 2], 2), gmean_us=round(gmean, 2), min_us=round(us[0], 2),
+                    p90_us=round(us[int(0.9 * (len(us) - 1))], 2), max_us=round(us[-1], 2),
+                    note="one call per event pair; event records sit inside each interval, so these run above the block mean")
 
     def time_cats_graph(t, steps, warmup):
         """The same steps replayed from a HIP graph holding one step per weight set."""
@@ -187,14 +246,25 @@ def main():
         us_graph, graph_steps = None, 0
     else:
         us_graph, graph_steps = time_cats_graph(t50, args.steps, args.warmup)
-    us_gate_up = time_cats(t50, args.steps, args.warmup, stages=1)
-    us_down = time_cats(t50, args.steps, args.warmup, stages=2)
+    us_k1 = time_cats(t50, args.steps, args.warmup, stage=1)
+    us_k2 = time_cats(t50, args.steps, args.warmup, stage=2)
+    rep_stats = per_rep_stats(t50, min(400, max(50, args.steps)))
     us_dense = time_dense(args.steps, args.warmup)
     us = us_eager if us_graph is None else min(us_eager, us_graph)
     launch = "stream" if (us_graph is None or us_eager <= us_graph) else "hipgraph"
     steps_timed = args.steps if launch == "stream" else graph_steps
     tb = touched_bytes(sz, B, k50)
-    b_gu, b_dn = stage_bytes(sz, B, k50)
+    single_pass = args.path != 1
+    if single_pass:
+        b_k1, b_k2 = stage_bytes(sz, B, k50)
+        k1_name = "cats::mlp_fused_kernel<F16,B=1> (gate GEMV + SiLU + threshold + sparse up + sparse down into per-workgroup partial sums)"
+        k2_name = "cats::reduce_partials_kernel<F16> (sum of the 256 partial sums, rounding, y)"
+    else:
+        b_k1 = sz * H * I + sz * H * k50 + sz * B * H + I // 8 + 4 * B * k50
+        b_k2 = sz * H * k50 + 4 * B * k50 + I // 8 + sz * B * H
+        k1_name = "cats::rows_kernel<F16,B=1,kGateUp> (gate GEMV + SiLU + threshold + sparse up)"
+        k2_name = "cats::down_kernel<F16,B=1> (sparse neuron-major down)"
+    traffic, traffic_note = measured_traffic() if (single_pass and abs(args.sparsity - 0.5) < 1e-9) else (None, "measured for the default path at 50 % only")
 
     sweep = []
     if not args.no_sweep:
@@ -234,20 +304,21 @@ def main():
         "dense_fp16_us": round(us_dense, 3),
         "dense_GBps": round(3 * sz * H * I / us_dense * 1e-3, 1),
         "speedup_vs_dense": round(us_dense / us, 3),
+        "per_rep": rep_stats,
         "roofline": {
             "bound": "hbm",
-            "kernel": "cats::rows_kernel<F16,B=1,kGateUp> (gate GEMV + SiLU + threshold + sparse up)",
-            "achieved": round(b_gu / us_gate_up * 1e-3, 1),
+            "kernel": k1_name,
+            "achieved": round(b_k1 / us_k1 * 1e-3, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
-            "frac": round(b_gu / us_gate_up * 1e-3 / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_HBM_BYTES_GATE_UP if abs(args.sparsity - 0.5) < 1e-9 else None,
-            "bytes_per_launch": int(b_gu),
-            "us_per_launch": round(us_gate_up, 3),
-            "second_kernel": {"kernel": "cats::down_kernel<F16,B=1> (sparse neuron-major down)", "bytes_per_launch": int(b_dn),
-                              "us_per_launch": round(us_down, 3), "achieved": round(b_dn / us_down * 1e-3, 1),
-                              "frac": round(b_dn / us_down * 1e-3 / HBM_PEAK_GBPS, 4)},
-            "note": "per-kernel times are back-to-back launches of that kernel alone (launch gap included); value is the whole call",
+            "frac": round(b_k1 / us_k1 * 1e-3 / HBM_PEAK_GBPS, 4),
+            "traffic": traffic,
+            "traffic_source": traffic_note,
+            "bytes_per_launch": int(b_k1),
+            "us_per_launch": round(us_k1, 3),
+            "second_kernel": {"kernel": k2_name, "bytes_per_launch": int(b_k2), "us_per_launch": round(us_k2, 3),
+                              "achieved": round(b_k2 / us_k2 * 1e-3, 1), "frac": round(b_k2 / us_k2 * 1e-3 / HBM_PEAK_GBPS, 4)},
+            "note": "per-kernel times are back-to-back launches of that kernel alone (launch gap included), timed with events on the launch stream; value is the whole call",
         },
         "sweep": sweep,
     }

@@ -22,7 +22,7 @@ DTYPE_CODE = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
 SYMBOLS = (
     "cats_version", "cats_status_string", "cats_workspace_bytes", "cats_workspace_init", "cats_gate_flag",
     "cats_gate_compact", "cats_read_count", "cats_up_flag", "cats_down_flag", "cats_gate_up", "cats_mlp",
-    "cats_mlp_rowmajor_down", "cats_mlp_norm_residual", "cats_up_down", "cats_set_tuning",
+    "cats_mlp_rowmajor_down", "cats_mlp_norm_residual", "cats_up_down", "cats_set_tuning", "cats_mlp_stage",
 )
 
 
@@ -52,6 +52,7 @@ def lib() -> ctypes.CDLL:
         L.cats_mlp_norm_residual.argtypes = [vp, vp, f32, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]
         L.cats_mlp_norm_residual.restype = i32
         L.cats_up_down.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_up_down.restype = i32
+        L.cats_mlp_stage.argtypes = [i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_mlp_stage.restype = i32
         L.cats_set_tuning.argtypes = [i32, i32, i32, i32]; L.cats_set_tuning.restype = i32
         _lib = L
     return _lib
@@ -183,5 +184,6 @@ def mlp_rowmajor_down(x, wgate, wup, wdown, threshold, ws: Workspace):
     return y
 
 
-def set_tuning(gate_variant=0, down_groups=0, down_block=0, stages=0):
-    lib().cats_set_tuning(int(gate_variant), int(down_groups), int(down_block), int(stages))
+def set_tuning(gate_variant=0, down_groups=0, down_block=0, path=0):
+    """path=1 keeps the whole-MLP entry points on the separate gate+up and sparse-down kernels at every batch size."""
+    lib().cats_set_tuning(int(gate_variant), int(down_groups), int(down_block), int(path))

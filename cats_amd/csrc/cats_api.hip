@@ -16,12 +16,16 @@ template <> hipError_t launch_rows<F32>(int, int, const RowsArgs&, hipStream_t);
 template <> hipError_t launch_down<F16>(int, bool, const DownArgs&, int, hipStream_t);
 template <> hipError_t launch_down<BF16>(int, bool, const DownArgs&, int, hipStream_t);
 template <> hipError_t launch_down<F32>(int, bool, const DownArgs&, int, hipStream_t);
+template <> hipError_t launch_fused<F16>(int, int, int, const FusedArgs&, const ReduceArgs&, hipStream_t);
+template <> hipError_t launch_fused<BF16>(int, int, int, const FusedArgs&, const ReduceArgs&, hipStream_t);
+template <> hipError_t launch_fused<F32>(int, int, int, const FusedArgs&, const ReduceArgs&, hipStream_t);
 namespace {
 
 Tuning g_tuning = {0, 0, 0, 0};
 #ifdef CATS_TIMING
 long long* g_tbuf_rows = nullptr;
 long long* g_tbuf_down = nullptr;
+long long* g_tbuf_fused = nullptr;
 #endif
 
 constexpr int kMaxSlabs = 128;
@@ -206,6 +210,64 @@ int check_ws(const void* ws, size_t ws_bytes, int H, int I, WsLayout& l) {
   return CATS_OK;
 }
 
+int device_cus() {
+  static int cus = 0;  // every GPU of a node is the same part, so one query serves all
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus = n;
+  }
+  return cus;
+}
+
+constexpr int kFusedMaxGrid = 256;  // partials of 256 workgroups x 2 batch rows fit the workspace's partial-sum region
+
+// Whether the single-pass kernel covers this call, and with what launch shape: one workgroup per CU, each with an
+// equal, contiguous share of the neurons.
+bool fused_eligible(int B, int H, int I, int dtype, FusedArgs& f, int& grid) {
+  if (g_tuning.path == 1 || B > 2) return false;
+  const int vec = vec_elems(dtype);
+  memset(&f, 0, sizeof(f));
+  f.H = H; f.I = I; f.nb = B;
+  f.row_vecs = H / vec;
+  f.nch = (f.row_vecs + kWave - 1) / kWave;
+  if (f.row_vecs > kFusedMaxKV * kFusedDownWaves * kWave) return false;
+  int maxgrid = device_cus();
+  if (maxgrid > kFusedMaxGrid) maxgrid = kFusedMaxGrid;
+  int rpw = (I + maxgrid - 1) / maxgrid;
+  if (rpw < 2 * kFusedRowWaves) rpw = 2 * kFusedRowWaves;  // small matrices: fewer workgroups rather than idle row waves
+  grid = (I + rpw - 1) / rpw;
+  f.rpw = rpw;
+  const int bt = batch_template(B);
+  const size_t nchv = (size_t)(f.nch + kFusedCB - 1) / kFusedCB * kFusedCB * kWave;
+  const size_t lds = bt * nchv * 16 + (size_t)((rpw + 3) & ~3) * 4 + (size_t)rpw * bt * 4;
+  return lds <= 128 * 1024;
+}
+
+int do_fused(FusedArgs& f, int grid, int stage, void* y_out, const void* residual, int32_t* count_out, int dtype, char* ws,
+             const WsLayout& l, hipStream_t s) {
+  f.partial = (float*)(ws + l.partial);
+  f.counts = (int32_t*)(ws + l.z32);
+#ifdef CATS_TIMING
+  f.tbuf = g_tbuf_fused;
+#endif
+  ReduceArgs r;
+  memset(&r, 0, sizeof(r));
+  r.partial = f.partial;
+  r.counts = f.counts;
+  r.y_out = y_out;
+  r.residual = residual;
+  r.count_out = count_out;
+  r.G = grid;
+  r.BH = f.nb * f.H;
+  const int bt = batch_template(f.nb);
+  hipError_t e;
+  if (dtype == CATS_F16) e = launch_fused<F16>(bt, grid, stage, f, r, s);
+  else if (dtype == CATS_BF16) e = launch_fused<BF16>(bt, grid, stage, f, r, s);
+  else e = launch_fused<F32>(bt, grid, stage, f, r, s);
+  return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+}
+
 }  // namespace
 }  // namespace cats
 
@@ -230,6 +292,7 @@ extern "C" {
 
 #ifdef CATS_TIMING
 void cats_timing_buffers(void* rows, void* down) { g_tbuf_rows = (long long*)rows; g_tbuf_down = (long long*)down; }
+void cats_timing_buffer_fused(void* fused) { g_tbuf_fused = (long long*)fused; }
 #endif
 
 int cats_version(void) { return 100; }
@@ -248,11 +311,11 @@ const char* cats_status_string(int status) {
   return "unknown status";
 }
 
-int cats_set_tuning(int gate_variant, int down_groups, int down_block, int stages) {
+int cats_set_tuning(int gate_variant, int down_groups, int down_block, int path) {
   g_tuning.gate_variant = gate_variant;
   g_tuning.down_groups = down_groups;
   g_tuning.down_block = down_block;
-  g_tuning.stages = stages;
+  g_tuning.path = path;
   return CATS_OK;
 }
 
@@ -361,7 +424,7 @@ static int gate_up_pass(const void* x, const void* wgate, const void* wup, void*
 
 static int mlp_pass(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, float* y_f32,
              uint8_t* flag_out, int32_t* count_out, int B, int H, int I, int dtype, float threshold, void* ws,
-             size_t ws_bytes, void* stream) {
+             size_t ws_bytes, void* stream, int stage = 0) {
   int st = check_common(B, H, I, dtype);
   if (st) return st;
   if (!x || !wgate || !wup || !wdown_t || ((y_f32 == nullptr) == (y_out == nullptr))) return CATS_ERR_NULL;
@@ -369,6 +432,17 @@ static int mlp_pass(const void* x, const void* wgate, const void* wup, const voi
   WsLayout l;
   st = check_ws(ws, ws_bytes, H, I, l);
   if (st) return st;
+  FusedArgs f;
+  int grid = 0;
+  if (y_out && fused_eligible(B, H, I, dtype, f, grid)) {
+    f.x = (const u32x4*)x;
+    f.wg = (const u32x4*)wgate;
+    f.wu = (const u32x4*)wup;
+    f.wd = (const u32x4*)wdown_t;
+    f.flag_out = flag_out;
+    f.t = round_through(dtype, threshold);
+    return do_fused(f, grid, stage, y_out, nullptr, count_out, dtype, (char*)ws, l, (hipStream_t)stream);
+  }
   RowsArgs a;
   fill_rows(a, x, wgate, H, I, B, dtype);
   a.w2 = (const u32x4*)wup;
@@ -376,11 +450,11 @@ static int mlp_pass(const void* x, const void* wgate, const void* wup, const voi
   a.mask_out = (uint8_t*)ws + l.mask;
   a.flag_out = flag_out;
   a.t = round_through(dtype, threshold);
-  if (g_tuning.stages != 2) {
+  if (stage != 2) {
     st = do_rows(kGateUp, dtype, a, (hipStream_t)stream);
     if (st) return st;
   }
-  if (g_tuning.stages == 1) return CATS_OK;
+  if (stage == 1) return CATS_OK;
   float* acc = y_f32;
   return do_down(a.z32_out, true, wdown_t, acc, y_out, count_out, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
 }
@@ -394,6 +468,16 @@ static int up_down_pass(const void* x, const void* a_in, const void* wup, const 
   WsLayout l;
   st = check_ws(ws, ws_bytes, H, I, l);
   if (st) return st;
+  FusedArgs f;
+  int grid = 0;
+  if (fused_eligible(B, H, I, dtype, f, grid)) {
+    f.x = (const u32x4*)x;
+    f.a_in = a_in;
+    f.wu = (const u32x4*)wup;
+    f.wd = (const u32x4*)wdown_t;
+    f.t = round_through(dtype, threshold);
+    return do_fused(f, grid, 0, y_out, nullptr, nullptr, dtype, (char*)ws, l, (hipStream_t)stream);
+  }
   RowsArgs a;
   fill_rows(a, x, wup, H, I, B, dtype);
   a.a_in = a_in;
@@ -418,6 +502,18 @@ static int mlp_norm_residual_pass(const void* h, const void* norm_weight, float 
   WsLayout l;
   st = check_ws(ws, ws_bytes, H, I, l);
   if (st) return st;
+  FusedArgs f;
+  int grid = 0;
+  if (fused_eligible(B, H, I, dtype, f, grid)) {
+    f.x = (const u32x4*)h;
+    f.wg = (const u32x4*)wgate;
+    f.wu = (const u32x4*)wup;
+    f.wd = (const u32x4*)wdown_t;
+    f.t = round_through(dtype, threshold);
+    f.norm_w = (const u32x4*)norm_weight;
+    f.norm_eps = eps;
+    return do_fused(f, grid, 0, out, h, nullptr, dtype, (char*)ws, l, (hipStream_t)stream);
+  }
   RowsArgs a;
   fill_rows(a, h, wgate, H, I, B, dtype);
   a.w2 = (const u32x4*)wup;
@@ -504,6 +600,13 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
     return mlp_pass(at_cbytes(x, b0 * H * sz), wgate, wup, wdown_t, at_bytes(y_out, b0 * H * sz), (float*)at_bytes((void*)y_f32, b0 * H * 4),
                     (uint8_t*)at_bytes((void*)flag_out, b0 * I), count_out, nb, H, I, dtype, threshold, ws, ws_bytes, stream);
   });
+}
+
+int cats_mlp_stage(int stage, const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,
+                   int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
+  if (stage != 1 && stage != 2) return CATS_ERR_SHAPE;
+  if (B > kKernelBatch) return CATS_ERR_BATCH;
+  return mlp_pass(x, wgate, wup, wdown_t, y_out, nullptr, nullptr, nullptr, B, H, I, dtype, threshold, ws, ws_bytes, stream, stage);
 }
 
 int cats_up_down(const void* x, const void* a, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,

@@ -286,6 +286,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   }
 
   if (p.count_out && blockIdx.x == 0) {  // not on the hot path: total popcount of the mask
+    __syncthreads();  // s_red is reused below; the fold above may still be reading it
     int k = 0;
     for (int byte = tid; byte * 8 < p.I; byte += blockDim.x) {
       uint32_t bits = p.mask[byte];

@@ -1,0 +1,462 @@
+// Whole CATS MLP in one streaming launch plus a small reduction launch, for 1 or 2 batch rows.
+//
+//   mlp_fused_kernel   One persistent workgroup of 16 waves per CU owns a contiguous range of neurons.  Eight "row
+//                      waves" take the range's neurons one at a time (LDS ticket): gate row -> SiLU -> threshold, and
+//                      for an active neuron the matching W_up row -> z.  The result of every neuron is published in an
+//                      LDS slot (dead, or live with its z).  Eight "down waves" own an eighth of the output columns
+//                      each; they walk the slots in neuron order and, for every live one, stream their part of that
+//                      neuron's W_down^T row into fp32 accumulators.  Nothing crosses a workgroup boundary while the
+//                      weights stream: no mask or z round trip through memory, no arrival counters, no second launch
+//                      ramp between the up and the down pass.  Each workgroup ends by storing its (nb, H) partial sums.
+//   reduce_partials_kernel  adds the per-workgroup partials in workgroup order, rounds to the storage type, optionally
+//                      adds the residual, writes y, and totals the per-workgroup active counts.
+//
+// Summation order is fixed (neurons ascending inside a workgroup, workgroups ascending in the reduction), so y is
+// bitwise reproducible run to run.  The two kernels are ordered by the stream, which is the only cross-workgroup
+// synchronisation there is.
+//
+// Inside the workgroup the producer / consumer hand-off runs through LDS: a row wave writes z, then the slot state;
+// the LDS unit executes one wave's accesses in issue order, so a down wave that reads "live" and then z reads the z
+// that was written before it.  Down waves poll with s_sleep; all waves of a workgroup are resident together, so the
+// producers always make progress.
+#pragma once
+#include "cats_device.h"
+
+namespace cats {
+
+constexpr int kFusedWaves = 16;
+constexpr int kFusedDownWaves = 8;
+constexpr int kFusedRowWaves = kFusedWaves - kFusedDownWaves;
+constexpr int kFusedThreads = kFusedWaves * kWave;
+constexpr int kFusedCB = 8;             // 64-lane chunks (of 16 bytes per lane) per block of row loads
+constexpr int kFusedMaxKV = 4;          // a down wave covers KV * 64 vectors of a row: rows of up to 4 * 8 * 64 vectors
+constexpr int kReduceCols = 32;         // fp32 columns per workgroup of the reduction kernel
+constexpr int kReduceLanes = 32;        // ranges of partials summed side by side per column
+
+enum FusedSlot { kSlotPending = 0, kSlotDead = 1, kSlotLive = 2 };
+
+struct FusedArgs {
+  const u32x4* x;        // (nb, H)
+  const u32x4* wg;       // (I, H); NULL when the gate activations are given (a_in)
+  const u32x4* wu;       // (I, H)
+  const u32x4* wd;       // (I, H) neuron-major
+  const void* a_in;      // optional (nb, I) dtype: gate activations; flags = |a| > t
+  uint8_t* flag_out;     // optional (nb, I)
+  float* partial;        // [grid][nb][H] fp32
+  int32_t* counts;       // [grid] live neurons per workgroup
+  const u32x4* norm_w;   // optional (H,) RMS-norm weight applied to x while it is staged
+  float norm_eps;
+  int H, I, nb;
+  int nch;               // 64-lane vector chunks per row: ceil(row_vecs / 64)
+  int row_vecs;          // H / VEC
+  int rpw;               // neurons per workgroup
+  float t;               // threshold, already rounded through dtype
+#ifdef CATS_TIMING
+  long long* tbuf;       // [gridDim][8] wall-clock stamps (100 MHz), development builds only
+#endif
+};
+
+struct ReduceArgs {
+  const float* partial;  // [G][BH]
+  const int32_t* counts; // [G]
+  void* y_out;           // (nb, H) dtype, flattened to BH
+  const void* residual;  // optional (nb, H) dtype; may alias y_out
+  int32_t* count_out;    // optional
+  int G;                 // number of partials
+  int BH;                // nb * H
+};
+
+#ifdef CATS_TIMING
+#define CATS_FSTAMP(cond, slot) do { if (p.tbuf && (cond)) p.tbuf[(size_t)blockIdx.x * 8 + (slot)] = wall_clock64(); } while (0)
+#else
+#define CATS_FSTAMP(cond, slot) do { } while (0)
+#endif
+
+// CB chunks of one row: 64 lanes x 16 bytes each, issued back to back.  Never predicated: lanes past the end of a
+// short row re-read its last vector and meet a zero in the LDS copy of x.
+template <int CB, bool FULL>
+__device__ __forceinline__ void fused_issue(const u32x4* __restrict__ row, int c0, int vlast, int lane, u32x4 (&wv)[CB]) {
+#pragma unroll
+  for (int cc = 0; cc < CB; cc++) {
+    const int v = (c0 + cc) * kWave + lane;
+    wv[cc] = load_stream(row + (FULL ? v : min(v, vlast)));
+  }
+}
+
+template <class DT, int B, int CB>
+__device__ __forceinline__ void fused_dot(const u32x4 (&wv)[CB], const u32x4* xs, int nchv, int c0, int lane, float (&acc)[B]) {
+#pragma unroll
+  for (int cc = 0; cc < CB; cc++) {
+    const int v = (c0 + cc) * kWave + lane;
+#pragma unroll
+    for (int b = 0; b < B; b++) acc[b] = DT::dot(wv[cc], xs[b * nchv + v], acc[b]);
+  }
+}
+
+// One batch of the down pass: RB row slots of KV vectors each.  The number of loads is fixed -- a slot without a row
+// reads one cached vector, the same address in every lane -- so the compiler can count loads in flight and wait for
+// exactly the older batch while the newer one stays outstanding.
+template <int B, int KV, int RB>
+struct DownBatch {
+  int rows[RB];       // neuron index, -1 = empty slot
+  float zz[RB][B];
+  int cnt;
+  u32x4 wv[RB][KV];
+};
+
+// Where the down waves read what the row waves publish: slot i is neuron row0 + i.
+struct FusedSlots {
+  volatile int* state;    // [n] FusedSlot
+  volatile float* z;      // [n][B]
+  int row0, n;
+};
+
+// Fill the batch with the next live neurons whose slots are published, in neuron order.  Blocking: wait until at
+// least one is there or the range is exhausted.  Non-blocking: take what is there, possibly nothing.
+// The wave looks at 64 slots per pass -- lane i reads state and z of slot head + i, ballots find the decided prefix and
+// the live slots in it -- so a pass costs one LDS round trip however many dead slots it steps over.
+template <int B, int KV, int RB>
+__device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const FusedSlots& sl, int& head, bool blocking) {
+  bt.cnt = 0;
+#pragma unroll
+  for (int u = 0; u < RB; u++) {
+    bt.rows[u] = -1;
+#pragma unroll
+    for (int b = 0; b < B; b++) bt.zz[u][b] = 0.f;
+  }
+  const int lane = threadIdx.x & (kWave - 1);
+  while (head < sl.n) {
+    const int idx = head + lane;
+    const bool in = idx < sl.n;  // never read past the slot array
+    const int st_ = in ? sl.state[idx] : kSlotPending;  // past the end counts as pending: it ends the decided prefix
+    int zv[B];
+#pragma unroll
+    for (int b = 0; b < B; b++) zv[b] = in ? __builtin_bit_cast(int, sl.z[idx * B + b]) : 0;
+    const uint64_t pend = __ballot(st_ == kSlotPending);
+    uint64_t live = __ballot(st_ == kSlotLive);
+    const int ready = pend ? __builtin_ctzll(pend) : kWave;  // slots head .. head + ready - 1 are decided
+    if (ready == 0) {
+      if (!blocking) return;
+      __builtin_amdgcn_s_sleep(1);
+      continue;
+    }
+    if (ready < kWave) live &= (1ull << ready) - 1ull;
+#pragma unroll
+    for (int u = 0; u < RB; u++) {
+      if (live) {  // uniform
+        const int bit = __builtin_ctzll(live);
+        live &= live - 1ull;
+        bt.rows[u] = sl.row0 + head + bit;
+#pragma unroll
+        for (int b = 0; b < B; b++) bt.zz[u][b] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zv[b], bit));
+        bt.cnt++;
+      }
+    }
+    head += live ? __builtin_ctzll(live) : ready;  // up to the first live slot that did not fit, else past the decided prefix
+    if (bt.cnt > 0) return;
+    // only dead slots so far: keep going
+  }
+}
+
+template <int B, int KV, int RB>
+__device__ __forceinline__ void fused_down_issue(DownBatch<B, KV, RB>& bt, const u32x4* __restrict__ wd, int row_vecs, const u32x4* dummy,
+                                                 const int (&vidx)[KV]) {
+#pragma unroll
+  for (int u = 0; u < RB; u++) {
+    const bool live = bt.rows[u] >= 0;  // uniform
+    const u32x4* r = live ? wd + (size_t)bt.rows[u] * row_vecs : dummy;
+#pragma unroll
+    for (int k = 0; k < KV; k++) bt.wv[u][k] = load_stream(r + (live ? vidx[k] : 0));
+  }
+}
+
+template <class DT, int B, int KV, int RB>
+__device__ __forceinline__ void fused_down_consume(const DownBatch<B, KV, RB>& bt, float (&acc)[B][KV][DT::VEC]) {
+#pragma unroll
+  for (int u = 0; u < RB; u++) {
+    if (bt.rows[u] >= 0) {  // uniform; the multiply-adds of an empty slot are skipped, its load is not
+#pragma unroll
+      for (int k = 0; k < KV; k++)
+#pragma unroll
+        for (int b = 0; b < B; b++) DT::axpy(bt.wv[u][k], bt.zz[u][b], acc[b][k]);
+    }
+  }
+}
+
+template <class DT, int B, bool FULL, int KV>
+__global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
+  typedef typename DT::st st;
+  constexpr int CB = kFusedCB;
+  constexpr int VEC = DT::VEC;
+  constexpr int RW = kFusedRowWaves;
+  constexpr int RB = 8 / (KV * B) < 1 ? 1 : 8 / (KV * B);  // row slots per batch of a down wave; two batches are in flight
+  constexpr int kXPre = 2;  // x vectors per thread fetched ahead of the first weight block
+  extern __shared__ u32x4 s_fused[];
+  __shared__ int s_ticket;
+  __shared__ float s_scale[B];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nchp = (p.nch + CB - 1) / CB * CB;
+  const int nchv = nchp * kWave;        // padded vectors per staged x row
+  const int vlast = p.row_vecs - 1;
+  const int row0 = blockIdx.x * p.rpw;
+  const int n = min(p.rpw, p.I - row0);  // neurons of this workgroup (>= 1 by the launch shape)
+
+  u32x4* xs = s_fused;                                       // [B][nchv]
+  FusedSlots sl;
+  sl.state = (volatile int*)(s_fused + B * nchv);          // [rpw]
+  sl.z = (volatile float*)(sl.state + ((p.rpw + 3) & ~3));  // [rpw][B]
+  sl.row0 = row0;
+  sl.n = n;
+
+  CATS_FSTAMP(tid == 0, 0);
+  const bool is_row_wave = wave >= kFusedDownWaves;
+  const int rw = wave - kFusedDownWaves;
+  const bool gate = p.wg != nullptr;
+
+  // Position in the workgroup's range -> neuron, or -1 past the end.
+  auto neuron_of = [&](int q) -> int { return q < n ? row0 + q : -1; };
+
+  // Staging, written out once per role so that each role's loads are counted on their own: memory returns are
+  // counted in issue order, x goes out first, then (row waves) the first gate block, and only x is waited for before
+  // the LDS writes and the barrier -- the weight loads stay in flight across both.
+  auto stage = [&](auto&& issue_first) {
+    u32x4 xpre[kXPre];
+#pragma unroll
+    for (int k = 0; k < kXPre; k++) {
+      const int i = tid + k * kFusedThreads;
+      const int b = B == 1 ? 0 : i / nchv, v = i - b * nchv;
+      xpre[k] = zero4();
+      if (i < B * nchv && b < p.nb && v < p.row_vecs) xpre[k] = p.x[(size_t)b * p.row_vecs + v];
+    }
+    issue_first();
+#pragma unroll
+    for (int k = 0; k < kXPre; k++) {
+      const int i = tid + k * kFusedThreads;
+      if (i < B * nchv) xs[i] = xpre[k];
+    }
+    for (int i = tid + kXPre * kFusedThreads; i < B * nchv; i += kFusedThreads) {
+      const int b = i / nchv, v = i - b * nchv;
+      u32x4 val = zero4();
+      if (b < p.nb && v < p.row_vecs) val = p.x[(size_t)b * p.row_vecs + v];
+      xs[i] = val;
+    }
+    for (int i = tid; i < p.rpw; i += kFusedThreads) sl.state[i] = kSlotPending;
+    if (tid == 0) s_ticket = 2 * RW;  // the first two neurons of every row wave are fixed, the rest go by ticket
+    __syncthreads();
+    if (p.norm_w) {
+      // RMS norm of each batch row, in place in LDS: one wave adds a row's squares (fixed order), everyone rescales.
+      for (int b = wave; b < B; b += kFusedWaves) {
+        float ss = 0.f;
+        for (int v = lane; v < p.row_vecs; v += kWave) ss = vec_sumsq<DT>(xs[b * nchv + v], ss);
+        ss = wave_sum(ss);
+        if (lane == 0) s_scale[b] = rsqrtf(ss / (float)p.H + p.norm_eps);
+      }
+      __syncthreads();
+      for (int i = tid; i < B * nchv; i += kFusedThreads) {
+        const int b = B == 1 ? 0 : i / nchv, v = i - b * nchv;
+        if (b < p.nb && v < p.row_vecs) xs[i] = vec_norm_apply<DT>(xs[i], s_scale[b], p.norm_w[v]);
+      }
+      __syncthreads();
+    }
+    CATS_FSTAMP(tid == 0, 1);
+  };
+
+  if (is_row_wave) {
+    // ---- row waves: gate (or given activation) -> decision -> up -> publish ------------------------------------
+    // A wave holds its current neuron, the next one (whose first gate block it prefetches) and the ticket after that.
+    int cur = neuron_of(rw);
+    int nxt = neuron_of(rw + RW);
+    u32x4 wc[CB];
+    stage([&] {
+      const u32x4* src = (gate && cur >= 0) ? p.wg + (size_t)cur * p.row_vecs : p.x;
+      fused_issue<CB, FULL>(src, 0, vlast, lane, wc);
+    });
+    const int nblk = nchp / CB;
+    const st* ain = (const st*)p.a_in;
+    while (cur >= 0) {
+      int pend = 0;
+      if (lane == 0) pend = __hip_atomic_fetch_add(&s_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      const int row = cur;
+      float a[B];
+      bool act[B];
+      bool any = false;
+      if (gate) {
+        float g[B];
+#pragma unroll
+        for (int b = 0; b < B; b++) g[b] = 0.f;
+        for (int blk = 0; blk < nblk; blk++) {
+          // next block of this row, or the first block of the next row this wave will take (past the end: x, cached)
+          const bool more = blk + 1 < nblk;
+          const u32x4* src = more ? p.wg + (size_t)row * p.row_vecs : (nxt >= 0 ? p.wg + (size_t)nxt * p.row_vecs : p.x);
+          u32x4 wn[CB];
+          fused_issue<CB, FULL>(src, more ? (blk + 1) * CB : 0, vlast, lane, wn);
+          fused_dot<DT, B, CB>(wc, xs, nchv, blk * CB, lane, g);
+#pragma unroll
+          for (int cc = 0; cc < CB; cc++) wc[cc] = wn[cc];
+        }
+#pragma unroll
+        for (int b = 0; b < B; b++) {
+          const float gr = DT::rnd(wave_sum(g[b]));
+          a[b] = DT::rnd(gr / (1.f + expf(-gr)));
+          act[b] = b < p.nb && fabsf(a[b]) > p.t;
+          any = any || act[b];
+        }
+      } else {
+#pragma unroll
+        for (int b = 0; b < B; b++) {
+          const float av = b < p.nb ? DT::tof(ain[(size_t)b * p.I + row]) : 0.f;
+          act[b] = b < p.nb && fabsf(av) > p.t;
+          a[b] = av;
+          any = any || act[b];
+        }
+        any = __builtin_amdgcn_readfirstlane((int)any) != 0;
+      }
+      float z[B];
+#pragma unroll
+      for (int b = 0; b < B; b++) z[b] = 0.f;
+      if (any) {  // wave-uniform
+        float u[B];
+#pragma unroll
+        for (int b = 0; b < B; b++) u[b] = 0.f;
+        const u32x4* ur = p.wu + (size_t)row * p.row_vecs;
+        for (int blk = 0; blk < nblk; blk++) {
+          u32x4 wu[CB];
+          fused_issue<CB, FULL>(ur, blk * CB, vlast, lane, wu);
+          fused_dot<DT, B, CB>(wu, xs, nchv, blk * CB, lane, u);
+        }
+#pragma unroll
+        for (int b = 0; b < B; b++) {
+          const float ub = wave_sum(u[b]);
+          z[b] = act[b] ? DT::rnd(a[b] * DT::rnd(ub)) : 0.f;
+        }
+      }
+      if (lane == 0) {
+        if (p.flag_out) {
+#pragma unroll
+          for (int b = 0; b < B; b++)
+            if (b < p.nb) p.flag_out[(size_t)b * p.I + row] = act[b] ? 1 : 0;
+        }
+        const int slot = row - row0;
+#pragma unroll
+        for (int b = 0; b < B; b++) sl.z[slot * B + b] = z[b];
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): z is in LDS before the state says so
+        sl.state[slot] = any ? kSlotLive : kSlotDead;
+      }
+      cur = nxt;
+      nxt = neuron_of(__builtin_amdgcn_readfirstlane(pend));
+    }
+#ifdef CATS_TIMING
+    if (p.tbuf && lane == 0) atomicMax((unsigned long long*)&p.tbuf[(size_t)blockIdx.x * 8 + 2], (unsigned long long)wall_clock64());
+#endif
+    return;
+  }
+
+  // ---- down waves: walk the slots in neuron order, stream this wave's columns of every live neuron ----------------
+  stage([] {});
+  const int d = wave;
+  int vidx[KV];
+#pragma unroll
+  for (int k = 0; k < KV; k++) vidx[k] = min((k * kFusedDownWaves + d) * kWave + lane, vlast);
+  float acc[B][KV][VEC];
+#pragma unroll
+  for (int b = 0; b < B; b++)
+#pragma unroll
+    for (int k = 0; k < KV; k++)
+#pragma unroll
+      for (int e = 0; e < VEC; e++) acc[b][k][e] = 0.f;
+
+  int head = 0, nlive = 0;
+  DownBatch<B, KV, RB> ba, bb;
+  fused_collect<B, KV, RB>(ba, sl, head, true);
+  fused_down_issue<B, KV, RB>(ba, p.wd, p.row_vecs, p.x, vidx);
+  for (;;) {
+    if (ba.cnt == 0 && head >= n) break;
+    fused_collect<B, KV, RB>(bb, sl, head, ba.cnt == 0);
+    fused_down_issue<B, KV, RB>(bb, p.wd, p.row_vecs, p.x, vidx);
+    fused_down_consume<DT, B, KV, RB>(ba, acc);
+    nlive += ba.cnt;
+    if (bb.cnt == 0 && head >= n) break;
+    fused_collect<B, KV, RB>(ba, sl, head, bb.cnt == 0);
+    fused_down_issue<B, KV, RB>(ba, p.wd, p.row_vecs, p.x, vidx);
+    fused_down_consume<DT, B, KV, RB>(bb, acc);
+    nlive += bb.cnt;
+  }
+  CATS_FSTAMP(lane == 0 && d == 0, 3);
+
+  float* mypart = p.partial + (size_t)blockIdx.x * p.nb * p.H;
+#pragma unroll
+  for (int k = 0; k < KV; k++) {
+    const int v = (k * kFusedDownWaves + d) * kWave + lane;
+    if (v < p.row_vecs) {
+#pragma unroll
+      for (int b = 0; b < B; b++)
+        if (b < p.nb) {
+          float4* dst = (float4*)(mypart + (size_t)b * p.H + (size_t)v * VEC);
+#pragma unroll
+          for (int q = 0; q < VEC / 4; q++) {
+            float4 o = {acc[b][k][4 * q], acc[b][k][4 * q + 1], acc[b][k][4 * q + 2], acc[b][k][4 * q + 3]};
+            dst[q] = o;
+          }
+        }
+    }
+  }
+  if (d == 0 && lane == 0) p.counts[blockIdx.x] = nlive;
+  CATS_FSTAMP(lane == 0 && d == 0, 4);
+#ifdef CATS_TIMING
+  if (p.tbuf && lane == 0 && d == 0) p.tbuf[(size_t)blockIdx.x * 8 + 6] = nlive;
+#endif
+}
+
+// y[c] = round(sum over g of partial[g][c]) (+ residual[c]);  c runs over the nb * H flattened outputs.  A workgroup of
+// 256 threads owns kReduceCols columns: 8 threads x float4 across, 32 side by side over contiguous ranges of partials
+// (all loads of a range in flight together), then one thread per column adds the 32 range sums in order.
+template <class DT>
+__global__ __launch_bounds__(256) void reduce_partials_kernel(ReduceArgs p) {
+  typedef typename DT::st st;
+  __shared__ float s_sum[kReduceLanes][kReduceCols + 4];
+  const int tid = threadIdx.x;
+  constexpr int kQ = kReduceCols / 4;  // threads across: one float4 each
+  static_assert(kQ * kReduceLanes == 256, "one workgroup covers kReduceCols columns x kReduceLanes ranges");
+  const int cq = tid % kQ, gl = tid / kQ;
+  const int col = blockIdx.x * kReduceCols + cq * 4;
+  const int per = (p.G + kReduceLanes - 1) / kReduceLanes;
+  const int g0 = gl * per, g1 = min(p.G, g0 + per);
+  float4 s = {0.f, 0.f, 0.f, 0.f};
+  if (col < p.BH) {
+    constexpr int U = 8;
+    for (int g = g0; g < g1; g += U) {
+      float4 t[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) t[u] = *(const float4*)(p.partial + (size_t)min(g + u, g1 - 1) * p.BH + col);
+#pragma unroll
+      for (int u = 0; u < U; u++)
+        if (g + u < g1) { s.x += t[u].x; s.y += t[u].y; s.z += t[u].z; s.w += t[u].w; }
+    }
+  }
+  s_sum[gl][cq * 4 + 0] = s.x;
+  s_sum[gl][cq * 4 + 1] = s.y;
+  s_sum[gl][cq * 4 + 2] = s.z;
+  s_sum[gl][cq * 4 + 3] = s.w;
+  __syncthreads();
+  if (tid < kReduceCols) {
+    const int c = blockIdx.x * kReduceCols + tid;
+    if (c < p.BH) {
+      float tot = 0.f;
+#pragma unroll
+      for (int l = 0; l < kReduceLanes; l++) tot += s_sum[l][tid];
+      if (p.residual) tot = DT::rnd(tot) + DT::tof(((const st*)p.residual)[c]);
+      ((st*)p.y_out)[c] = DT::fromf(tot);
+    }
+  }
+  if (p.count_out && blockIdx.x == 0 && tid >= 64 && tid < 128) {  // second wave: total of the per-workgroup counts
+    int k = 0;
+    for (int g = tid - 64; g < p.G; g += kWave) k += p.counts[g];
+    k = (int)wave_sum((float)k);  // far below 2^24: exact in fp32
+    if (tid == 64) *p.count_out = k;
+  }
+}
+
+}  // namespace cats

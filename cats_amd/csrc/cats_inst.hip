@@ -127,7 +127,44 @@ hipError_t launch_down_one(const DownArgs& a, int block, hipStream_t stream) {
   return hipGetLastError();
 }
 
+template <class DT, int B, bool FULL, int KV>
+hipError_t launch_fused_one(int grid, const FusedArgs& a, hipStream_t stream) {
+  auto kern = mlp_fused_kernel<DT, B, FULL, KV>;
+  const int nchv = (a.nch + kFusedCB - 1) / kFusedCB * kFusedCB * kWave;
+  const size_t lds = (size_t)B * nchv * sizeof(u32x4) + (size_t)((a.rpw + 3) & ~3) * 4 + (size_t)a.rpw * B * 4;
+  if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kFusedThreads), lds, stream, a);
+  return hipGetLastError();
+}
+
+template <class DT, int B>
+hipError_t launch_fused_b(int grid, const FusedArgs& a, hipStream_t stream) {
+  const bool full = a.H % (kWave * DT::VEC * kFusedCB) == 0;
+  const int kv = (a.row_vecs + kFusedDownWaves * kWave - 1) / (kFusedDownWaves * kWave);
+#define CATS_FUSED_KV(KVV)                                                              \
+  if (kv <= KVV) return full ? launch_fused_one<DT, B, true, KVV>(grid, a, stream)      \
+                             : launch_fused_one<DT, B, false, KVV>(grid, a, stream);
+  CATS_FUSED_KV(1)
+  CATS_FUSED_KV(2)
+  CATS_FUSED_KV(4)
+#undef CATS_FUSED_KV
+  return hipErrorInvalidValue;
+}
+
 }  // namespace
+
+template <>
+hipError_t launch_fused<CATS_DT>(int bt, int grid, int stage, const FusedArgs& a, const ReduceArgs& r, hipStream_t stream) {
+  if (stage != 2) {
+    hipError_t e = bt == 1 ? launch_fused_b<CATS_DT, 1>(grid, a, stream) : launch_fused_b<CATS_DT, 2>(grid, a, stream);
+    if (e != hipSuccess) return e;
+  }
+  if (stage != 1) {
+    hipLaunchKernelGGL(reduce_partials_kernel<CATS_DT>, dim3((r.BH + kReduceCols - 1) / kReduceCols), dim3(256), 0, stream, r);
+    return hipGetLastError();
+  }
+  return hipSuccess;
+}
 
 template <>
 hipError_t launch_rows<CATS_DT>(int mode, int bt, const RowsArgs& a, hipStream_t stream) {

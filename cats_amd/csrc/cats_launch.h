@@ -3,6 +3,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include "cats_down.h"
+#include "cats_fused.h"
 #include "cats_rows.h"
 
 namespace cats {
@@ -11,7 +12,7 @@ struct Tuning {
   int gate_variant;  // N > 0: cap the rows kernel at N workgroups per CU (dynamic-LDS floor); 0 = no cap
   int down_groups;   // 0 = default (about one workgroup per CU over all slabs)
   int down_block;    // 0 = default (1024 threads)
-  int stages;        // cats_mlp only: 0 = both launches, 1 = gate+up only, 2 = down only (profiling)
+  int path;          // whole-MLP entry points: 0 = choose by shape, 1 = always the separate gate+up and down kernels
 };
 
 // Returns hipSuccess or the launch error.  `mode` is a RowsMode; bt (1, 2, 4 or 8) the compile-time batch.
@@ -20,5 +21,9 @@ hipError_t launch_rows(int mode, int bt, const RowsArgs& a, hipStream_t stream);
 
 template <class DT>
 hipError_t launch_down(int bt, bool zf32, const DownArgs& a, int block, hipStream_t stream);
+
+// Single-pass MLP for 1 or 2 batch rows.  stage: 0 = both launches, 1 = streaming kernel only, 2 = reduction only.
+template <class DT>
+hipError_t launch_fused(int bt, int grid, int stage, const FusedArgs& a, const ReduceArgs& r, hipStream_t stream);
 
 }  // namespace cats

@@ -7,6 +7,7 @@
 // status becomes a c10::Error (the reference printf()s and exit()s: fuse_gemv_cmp_cuda.cu:2096-2097).
 #include <ATen/ATen.h>
 #include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
 #include <torch/library.h>
 
 #include <map>
@@ -57,16 +58,25 @@ struct Workspace {
   size_t bytes = 0;
 };
 
-// One workspace per (device, stream, H, I): the carving of a workspace is tied to the layer shape.  It is
-// allocated and zero-filled (by a kernel on the calling stream) on the first call for a shape, so run one
-// call before capturing a HIP graph.
+// One workspace per (device, stream, H, I): the carving of a workspace is tied to the layer shape, and one workspace
+// serves one stream at a time.  It is allocated and zero-filled (by a kernel on the calling stream) on the first call
+// for a shape; that first call must not happen under stream capture (the allocation would come out of the graph's
+// private pool and the fill would be recorded into the graph), so it is refused there: run one call eagerly on the
+// capturing stream first.  A captured graph keeps using the workspace of the stream it was captured on, so eager
+// calls on that stream must not overlap its replays.  Entries live until the process ends (a few MB per layer shape
+// and stream; torch hands out at most 32 pooled side streams per device) and the map is never destroyed: at exit the
+// HIP runtime may be gone before static destructors run.
 Workspace& workspace(const at::Tensor& like, int B, int H, int I, hipStream_t stream) {
   static std::mutex mu;
-  static std::map<std::tuple<int, void*, int, int>, Workspace> cache;
+  static auto& cache = *new std::map<std::tuple<int, void*, int, int>, Workspace>();
   std::lock_guard<std::mutex> lock(mu);
   Workspace& ws = cache[std::make_tuple((int)like.get_device(), (void*)stream, H, I)];
   const size_t need = cats_workspace_bytes(B, H, I);
   if (ws.bytes < need) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    TORCH_CHECK(hipStreamIsCapturing(stream, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone,
+                "flash_gemv: the first call for a layer shape on a stream allocates its workspace and cannot run under "
+                "stream capture; call the op once on this stream before capturing");
     ws.buf = at::empty({(int64_t)need}, like.options().dtype(at::kByte));
     ws.bytes = need;
     check_status(cats_workspace_init(ws.buf.data_ptr(), need, stream), "workspace_init");
@@ -362,10 +372,6 @@ std::tuple<at::Tensor, at::Tensor, at::Tensor> cats_mlp_stats_op(const at::Tenso
   return {out, flags, count};
 }
 
-void cats_set_tuning_op(int64_t gate_variant, int64_t down_groups, int64_t down_block, int64_t stages) {
-  cats_set_tuning((int)gate_variant, (int)down_groups, (int)down_block, (int)stages);
-}
-
 }  // namespace
 
 TORCH_LIBRARY(flash_gemv, m) {
@@ -390,5 +396,4 @@ TORCH_LIBRARY(flash_gemv, m) {
   m.def("cats_mlp_norm_residual", cats_mlp_norm_residual_op);
   m.def("cats_up_down", cats_up_down_op);
   m.def("cats_mlp_stats", cats_mlp_stats_op);
-  m.def("cats_set_tuning", cats_set_tuning_op);
 }

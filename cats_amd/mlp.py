@@ -86,6 +86,7 @@ class CatsMLP(nn.Module):
         self.visit_counts = 0
         self.count = 0
         self.t = 0
+        self.decode_fetched: Optional[torch.Tensor] = None  # neurons fetched by the kernel path while is_stats (device int64)
         self.histogram_bins = histogram_bins()
         self.pre_act_hist_counts = torch.zeros(NUM_BINS - 1)
         self.post_act_hist_counts = torch.zeros(NUM_BINS - 1)
@@ -95,10 +96,18 @@ class CatsMLP(nn.Module):
         self.is_stats = True
         self.dead_percentage = 0
         self.visit_counts = 0
+        self.decode_fetched = None
         self.is_collect_histogram = is_collect_histogram
 
     def deactivate_stats(self):
         self.is_stats = False
+
+    def decode_union_sparsity(self) -> Optional[float]:
+        """1 - (neurons fetched per call) / I over the kernel-path calls made while is_stats; None if there were none.
+        This is what the reference's microbenchmark reports as sparsity (flash_gemv/bench/profile_llama7B.py:56,72)."""
+        if self.decode_fetched is None or self.visit_counts == 0:
+            return None
+        return 1.0 - float(self.decode_fetched.item()) / (self.visit_counts * self.intermediate_size)
 
     def collect_stats(self, pre_activation, post_activation):
         start_time = time.time()
@@ -152,6 +161,16 @@ class CatsMLP(nn.Module):
                     raise RuntimeError("CatsMLP: sp_method 2/3 need wdown_t (call prepare_decode() once after loading weights)")
                 if self.sp_method == 2:
                     return flash_gemv.gemv_gemv_triton(x, self.act_fn(self.gate_proj(x)), self.up_proj.weight, self.wdown_t, t)
+                if self.is_stats:
+                    # decode-time sparsity bookkeeping (the reference's agg_sparsity, ugly_utils.py:929-937, for the
+                    # kernel path): the kernel reports how many neurons it fetched -- the union over the rows -- and
+                    # the running total stays on the device, so nothing here waits for the GPU
+                    y, _, fetched = flash_gemv.cats_mlp_stats(x, self.gate_proj.weight, self.up_proj.weight, self.wdown_t, t)
+                    if self.decode_fetched is None or self.decode_fetched.device != fetched.device:
+                        self.decode_fetched = torch.zeros((), dtype=torch.int64, device=fetched.device)
+                    self.decode_fetched += fetched
+                    self.visit_counts += 1
+                    return y
                 return flash_gemv.cats_mlp(x, self.gate_proj.weight, self.up_proj.weight, self.wdown_t, t)
             return self._dense_masked(x)
 

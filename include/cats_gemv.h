@@ -111,7 +111,9 @@ int cats_down_flag(const void* z, const void* wdown_t, const uint8_t* flag, floa
 int cats_gate_up(const void* x, const void* wgate, const void* wup, void* out, uint8_t* flag_out,
                  int B, int H, int I, int dtype, float threshold, void* stream);
 
-/* Whole CATS MLP with neuron-major down weights: two launches (gate+up, sparse down).
+/* Whole CATS MLP with neuron-major down weights, two launches.  1..2 rows: one streaming kernel in which every workgroup
+ * takes its neurons through gate, up and down and leaves (B,H) partial sums, then a reduction over the workgroups;
+ * more rows (and y_f32 mode): gate+up kernel, then sparse down kernel.
  *   y_out != NULL : (B,H) in dtype;  y_f32 != NULL : fp32 accumulate into the caller's pre-zeroed (B,H).
  * flag_out (B,I) optional.  count_out (device int32, optional, B <= 8 only) receives the number of neurons fetched
  * (union over the batch).
@@ -148,12 +150,18 @@ int cats_mlp_norm_residual(const void* h, const void* norm_weight, float eps, co
 int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out,
                            int B, int H, int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream);
 
-/* Launch-shape knobs for experiments and profiling; 0 keeps the built-in choice.  gate_variant N > 0 caps the
- * gate / up kernel at N resident workgroups per CU; down_groups / down_block set the neuron groups and the
- * workgroup size of the sparse down kernel.  `stages` restricts cats_mlp
- * to one of its two launches (1 = gate+up only, 2 = sparse down only, over whatever mask and z the workspace
- * holds from the previous full call) so each kernel can be timed alone.  Process-global; not in the reference. */
-int cats_set_tuning(int gate_variant, int down_groups, int down_block, int stages);
+/* One launch of cats_mlp(y_out mode) alone, for per-kernel timing and profiling: stage 1 = the streaming launch (gate, up
+ * and, for 1..2 rows, down into per-workgroup partial sums), stage 2 = the launch that finishes y from what stage 1 left in
+ * the workspace.  Calling stage 1 then stage 2 with the same arguments is cats_mlp.  Not in the reference. */
+int cats_mlp_stage(int stage, const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out,
+                   int B, int H, int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream);
+
+/* Launch-shape knobs for experiments; 0 keeps the built-in choice.  gate_variant N > 0 caps the gate / up kernel at N
+ * resident workgroups per CU (N < 0 keeps 3..8 rows off the matrix-core kernel); down_groups / down_block set the neuron
+ * groups and the workgroup size of the sparse down kernel; path 1 keeps the whole-MLP entry points on the separate gate+up
+ * and sparse-down kernels for every batch size (by default 1..2 rows take the single-pass kernel).  Every setting computes
+ * the same function.  Process-global and not synchronised: set it before other threads call in.  Not in the reference. */
+int cats_set_tuning(int gate_variant, int down_groups, int down_block, int path);
 
 #ifdef __cplusplus
 }

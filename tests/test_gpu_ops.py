@@ -249,6 +249,41 @@ def test_decode_loop_with_fused_layer_tail():
     assert agree >= 0.9, f"only {agree:.2f} of the greedy tokens agree between the fused and the unfused layer tail"
 
 
+def test_full_size_decoder_parity_agreement_and_sparsity():
+    """The 32-layer 4096 / 11008 fp16 decoder of the end-to-end benchmark.
+    (1) Every MLP call of an 8-token decode, on the hidden states the model really produces: the HIP result against
+        the dense-masked formula on identical gate values, to rtol 1e-2 / atol 2e-3; flags bit-exact on the kernel's own
+        activations; flags against PyTorch's gate GEMV differing only within a rounding step of the threshold.
+    (2) Over 32 greedy tokens fed to every mode: the HIP modes stay as close to the dense-masked PyTorch model as that
+        model stays to itself when its thresholds move by 0.1 % (a random-init 32-layer network amplifies single mask
+        bits; that control measures by how much).  Bar: top-token agreement and logit distance no worse than twice
+        the control's disagreement / distance, and at least half of the top tokens the same.
+    (3) The sparsity the kernels met while decoding is within 5 points of the calibrated 50 % in every layer."""
+    from cats_amd import decoder as dec
+
+    cfg = dec.DecoderConfig(num_layers=32, max_len=128 + 40)
+    model = dec.LlamaDecoder(cfg, torch.float16, "cuda", seed=0).eval()
+    model.calibrate(0.5)
+    g = torch.Generator(device="cuda").manual_seed(7)
+    prompt = torch.randint(0, cfg.vocab_size, (1, 128), generator=g, device="cuda")
+    lw = dec.layerwise_parity(model, prompt, 8)
+    print(f"[full-size decode] layerwise {lw}", flush=True)
+    assert lw["mlp_calls_checked"] == 32 * 7
+    assert lw["calls_outside_tolerance"] == 0 and lw["flags_not_matching_own_activations"] == 0, lw
+    assert lw["mask_bits_differing_from_torch_gate"] <= 1e-3 * lw["mask_bits_total"], lw
+    assert lw["largest_distance_from_threshold_of_a_differing_bit"] <= 2e-3, lw   # one fp16 step at |a| ~ 0.26 is 2.4e-4
+    agree, sparsity = dec.compare_modes(model, prompt, 32)
+    print(f"[full-size decode] {agree} mean sparsity {sum(sparsity) / len(sparsity):.4f}", flush=True)
+    assert agree["self_consistent"]
+    floor = agree["cats_torch_nudged"]
+    for mode in ("cats", "cats_fused"):
+        assert agree[mode]["argmax_agreement"] >= max(0.5, 1 - 2 * (1 - floor["argmax_agreement"])), (mode, agree)
+        assert agree[mode]["max_logit_diff"] <= max(2 * floor["max_logit_diff"], 0.02 * floor["logit_scale"]), (mode, agree)
+    assert len(sparsity) == 32 and all(0.45 <= v <= 0.55 for v in sparsity), sparsity
+    del model
+    torch.cuda.empty_cache()
+
+
 def test_two_streams_with_their_own_workspaces_do_not_interfere():
     """Calls on different streams run concurrently on the GPU; each stream has its own workspace (counters, partial
     sums, mask), so results must equal those of the same calls run one after the other."""

@@ -394,6 +394,95 @@ def test_matrix_core_and_wave_per_row_kernels_agree(oracle):
         close(y_m.cpu(), y_w.cpu(), torch.float16)
 
 
+SINGLE_PASS = [
+    # H, I, B, dtype -- every template the single-pass kernel is instantiated for (row length in whole blocks of 512
+    # vectors or not, 1 / 2 / 4 vectors of a row per down wave), ranges that end short, fewer neurons than row waves
+    (4096, 11008, 1, torch.float16), (4096, 14336, 1, torch.bfloat16), (4096, 2048, 2, torch.float16),
+    (520, 1000, 2, torch.float16), (260, 333, 1, torch.float32), (8192, 1024, 1, torch.float16), (8192, 600, 2, torch.bfloat16),
+    (4096, 700, 1, torch.float32), (8192, 300, 1, torch.float32), (64, 96, 1, torch.float16), (72, 5, 2, torch.bfloat16), (2048, 4099, 2, torch.float32),
+]
+
+
+@pytest.mark.parametrize("H,I,B,dtype", SINGLE_PASS)
+def test_single_pass_and_two_kernel_paths_agree(oracle, H, I, B, dtype):
+    """cats_mlp for 1..2 rows runs as one streaming kernel + a reduction; the tuning knob puts the same call on the
+    separate gate+up and sparse-down kernels.  Same activations bit for bit (same dot-product order), so the same
+    flags and count; outputs agree to the parity tolerance; the single-pass result is bitwise repeatable."""
+    m = make_mlp(H, I, B, dtype, seed=H + 3 * I + B, corr=0.5 if B > 1 else 0.0)
+    d = dev(m)
+    ws = _ws(B, H, I)
+    a_abs = oracle.c_gate(m["x"], m["wg"], -1.0)[0].float().abs().flatten()
+    nw = (torch.rand(H) + 0.5).to(dtype).cuda()
+    for q in (0.0, 0.5, 0.93):
+        t = -1.0 if q == 0.0 else float(torch.quantile(a_abs, q))
+        print(f"[case] single-pass H={H} I={I} B={B} {dtype} q={q}", flush=True)
+        try:
+            capi.set_tuning(0, 0, 0, 1)
+            y2, f2, c2 = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
+            n2 = capi.mlp_norm_residual(d["x"], nw, 1e-5, d["wg"], d["wu"], d["wdt"], t, ws)
+            a, _ = capi.gate_flag(d["x"], d["wg"], t)
+            u2 = capi.up_down(d["x"], a, d["wu"], d["wdt"], t, ws)
+            torch.cuda.synchronize()
+        finally:
+            capi.set_tuning(0, 0, 0, 0)
+        y1, f1, c1 = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
+        y1b = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws)
+        n1 = capi.mlp_norm_residual(d["x"], nw, 1e-5, d["wg"], d["wu"], d["wdt"], t, ws)
+        u1 = capi.up_down(d["x"], a, d["wu"], d["wdt"], t, ws)
+        torch.cuda.synchronize()
+        assert torch.equal(f1, f2) and int(c1) == int(c2) == int(f1.any(dim=0).sum())
+        assert torch.equal(y1, y1b), "single-pass output differs between two calls"
+        close(y1.cpu(), y2.cpu(), dtype)
+        close(u1.cpu(), u2.cpu(), dtype)
+        close(u1.cpu(), y2.cpu(), dtype)
+        # the folded norm changes x in its last bits between kernels' staging paths: same tolerance, on the residual sum
+        close(n1.cpu(), n2.cpu(), dtype)
+        ref = oracle.c_mlp(m["x"], m["wg"], m["wu"], m["wd"], t, a_in=a.cpu(), flag_in=f1.cpu())
+        close(y1.cpu(), ref["y"], dtype)
+
+
+def test_mlp_stage_launches_compose_to_the_whole_call():
+    """cats_mlp_stage(1) then cats_mlp_stage(2) is cats_mlp, on the single-pass path (1 row) and on the two-kernel path (4 rows)."""
+    import ctypes
+
+    L = capi.lib()
+    for B in (1, 4):
+        m = make_mlp(4096, 1536, B, torch.float16, seed=5 + B)
+        d = dev(m)
+        t = calibrate(m["wg"], [0.5])[0]
+        ws = _ws(B, 4096, 1536)
+        want = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws)
+        got = torch.zeros_like(want)
+        p = lambda x: ctypes.c_void_p(x.data_ptr())
+        s = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        for stage in (1, 2):
+            capi.check(L.cats_mlp_stage(stage, p(d["x"]), p(d["wg"]), p(d["wu"]), p(d["wdt"]), p(got), B, 4096, 1536, capi.F16,
+                                        ctypes.c_float(t), p(ws.buf), ws.nbytes, s), "cats_mlp_stage")
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+    assert L.cats_mlp_stage(3, None, None, None, None, None, 1, 64, 64, 0, ctypes.c_float(0), None, 0, None) != 0
+
+
+@pytest.mark.parametrize("B", [1, 2, 4])
+def test_active_count_does_not_disturb_the_down_kernel_output(B):
+    """The sparse down kernel totals the mask in the LDS it has just folded its partial sums through: asking for the
+    count must not change a single output bit."""
+    m = make_mlp(4096, 4096, B, torch.float16, seed=91 + B, corr=0.5)
+    d = dev(m)
+    t = calibrate(m["wg"], [0.5])[0]
+    ws = _ws(B, 4096, 4096)
+    try:
+        capi.set_tuning(0, 0, 0, 1)  # two-kernel path at every batch size
+        y_plain = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws)
+        for _ in range(5):
+            y_cnt, flag, cnt = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
+            torch.cuda.synchronize()
+            assert torch.equal(y_cnt, y_plain)
+            assert int(cnt) == int(flag.any(dim=0).sum())
+    finally:
+        capi.set_tuning(0, 0, 0, 0)
+
+
 def _gap_threshold(a_abs, q):
     """A threshold near the q-quantile of |a| that sits in the middle of the widest gap between neighbouring values
     there, so that a last-bit difference in the normalised input cannot move a neuron across it."""
