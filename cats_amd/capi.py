@@ -22,7 +22,7 @@ DTYPE_CODE = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
 SYMBOLS = (
     "cats_version", "cats_status_string", "cats_workspace_bytes", "cats_workspace_init", "cats_gate_flag",
     "cats_gate_compact", "cats_read_count", "cats_up_flag", "cats_down_flag", "cats_gate_up", "cats_mlp",
-    "cats_mlp_rowmajor_down", "cats_mlp_norm_residual", "cats_up_down", "cats_set_tuning", "cats_mlp_stage",
+    "cats_mlp_rowmajor_down", "cats_mlp_norm_residual", "cats_up_down", "cats_set_tuning", "cats_mlp_stage", "cats_mlp_noalloc",
 )
 
 
@@ -53,6 +53,7 @@ def lib() -> ctypes.CDLL:
         L.cats_mlp_norm_residual.restype = i32
         L.cats_up_down.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_up_down.restype = i32
         L.cats_mlp_stage.argtypes = [i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_mlp_stage.restype = i32
+        L.cats_mlp_noalloc.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp]; L.cats_mlp_noalloc.restype = i32
         L.cats_set_tuning.argtypes = [i32, i32, i32, i32]; L.cats_set_tuning.restype = i32
         _lib = L
     return _lib
@@ -154,6 +155,14 @@ def mlp(x, wgate, wup, wdown_t, threshold, ws: Workspace, y=None, want_flag=Fals
     if want_flag or want_count:
         return out, flag, count
     return out
+
+
+def mlp_noalloc(x, wgate, wup, wdown_t, threshold, y):
+    """cats_mlp into the caller's y with the library's built-in scratch: no workspace, nothing allocated by the call."""
+    B, H, I = _dims(x, wgate)
+    check(lib().cats_mlp_noalloc(_p(x), _p(wgate), _p(wup), _p(wdown_t), _p(y), B, H, I, DTYPE_CODE[x.dtype], float(threshold),
+                                 _stream(x)), "cats_mlp_noalloc")
+    return y
 
 
 def up_down(x, a, wup, wdown_t, threshold, ws: Workspace):

@@ -4,8 +4,16 @@
 #include <hip/hip_runtime.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "cats_gemv.h"
 #include "cats_launch.h"
+
+// Built-in scratch of cats_mlp_noalloc: the per-workgroup partial sums and active counts of the single-pass kernel.
+// Every GPU the library runs on holds its own copy of this array, at its own address, until the process ends.
+constexpr size_t kScratchPartialBytes = (size_t)256 * 8192 * 4;  // 256 workgroups x (B * H <= 8192) fp32 partial sums
+constexpr size_t kScratchBytes = kScratchPartialBytes + 4096;    // + one int32 count per workgroup
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 namespace cats {
 
@@ -268,6 +276,28 @@ int do_fused(FusedArgs& f, int grid, int stage, void* y_out, const void* residua
   return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
 }
 
+// Device address of this GPU's copy of `scratch`.  The array's name means nothing to a kernel when it is used in host
+// code, so the address is asked for once per device (with that device current) and kept.
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mu;
+
+int scratch_address(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return CATS_ERR_LAUNCH;
+  void* p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (p == nullptr) {
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    p = g_scratch_ptr[dev];
+    if (p == nullptr) {
+      if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return CATS_ERR_LAUNCH;
+      __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);
+    }
+  }
+  *out = p;
+  return CATS_OK;
+}
+
 }  // namespace
 }  // namespace cats
 
@@ -307,6 +337,7 @@ const char* cats_status_string(int status) {
     case CATS_ERR_NULL: return "required pointer is NULL";
     case CATS_ERR_WORKSPACE: return "workspace missing, misaligned (256 bytes) or smaller than cats_workspace_bytes()";
     case CATS_ERR_LAUNCH: return "HIP kernel launch failed";
+    case CATS_ERR_SCRATCH: return "call does not fit the built-in scratch of cats_mlp_noalloc (1..2 rows, B * H <= 8192, rows of at most 2048 16-byte vectors)";
   }
   return "unknown status";
 }
@@ -607,6 +638,46 @@ int cats_mlp_stage(int stage, const void* x, const void* wgate, const void* wup,
   if (stage != 1 && stage != 2) return CATS_ERR_SHAPE;
   if (B > kKernelBatch) return CATS_ERR_BATCH;
   return mlp_pass(x, wgate, wup, wdown_t, y_out, nullptr, nullptr, nullptr, B, H, I, dtype, threshold, ws, ws_bytes, stream, stage);
+}
+
+int cats_mlp_noalloc(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,
+                     int dtype, float threshold, void* stream) {
+  int st = check_common(B, H, I, dtype);
+  if (st) return st;
+  if (!x || !wgate || !wup || !wdown_t || !y_out) return CATS_ERR_NULL;
+  if (!aligned16(x) || !aligned16(wgate) || !aligned16(wup) || !aligned16(wdown_t)) return CATS_ERR_ALIGN;
+  FusedArgs f;
+  int grid = 0;
+  const int saved_path = g_tuning.path;
+  g_tuning.path = 0;  // this entry point is the single-pass kernel or nothing
+  const bool ok = fused_eligible(B, H, I, dtype, f, grid);
+  g_tuning.path = saved_path;
+  // the stated limit (B * H <= 8192) whatever the grid turns out to be, and the actual footprint as a second check
+  if (!ok || (size_t)B * H > 8192 || (size_t)grid * B * H * 4 > kScratchPartialBytes || (size_t)grid * 4 > kScratchBytes - kScratchPartialBytes)
+    return CATS_ERR_SCRATCH;
+  void* sp = nullptr;
+  st = scratch_address(&sp);
+  if (st) return st;
+  f.x = (const u32x4*)x;
+  f.wg = (const u32x4*)wgate;
+  f.wu = (const u32x4*)wup;
+  f.wd = (const u32x4*)wdown_t;
+  f.t = round_through(dtype, threshold);
+  f.partial = (float*)sp;
+  f.counts = (int32_t*)((char*)sp + kScratchPartialBytes);
+  ReduceArgs r;
+  memset(&r, 0, sizeof(r));
+  r.partial = f.partial;
+  r.counts = f.counts;
+  r.y_out = y_out;
+  r.G = grid;
+  r.BH = B * H;
+  const int bt = batch_template(B);
+  hipError_t e;
+  if (dtype == CATS_F16) e = launch_fused<F16>(bt, grid, 0, f, r, (hipStream_t)stream);
+  else if (dtype == CATS_BF16) e = launch_fused<BF16>(bt, grid, 0, f, r, (hipStream_t)stream);
+  else e = launch_fused<F32>(bt, grid, 0, f, r, (hipStream_t)stream);
+  return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
 }
 
 int cats_up_down(const void* x, const void* a, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,

@@ -50,7 +50,8 @@ typedef enum {
   CATS_ERR_BATCH = 4,      /* B outside 1..CATS_MAX_BATCH */
   CATS_ERR_NULL = 5,       /* a required pointer is NULL */
   CATS_ERR_WORKSPACE = 6,  /* workspace missing or smaller than cats_workspace_bytes() */
-  CATS_ERR_LAUNCH = 7      /* the HIP runtime refused a launch; hipGetLastError() has details */
+  CATS_ERR_LAUNCH = 7,     /* the HIP runtime refused a launch; hipGetLastError() has details */
+  CATS_ERR_SCRATCH = 8     /* cats_mlp_noalloc: the call does not fit the library's built-in scratch */
 } cats_status_t;
 
 #define CATS_MAX_BATCH 16  /* 1..8 rows are one pass over the weights; 9..16 rows are two (the weights are read per pass) */
@@ -149,6 +150,18 @@ int cats_mlp_norm_residual(const void* h, const void* norm_weight, float eps, co
  * fuse_gemv_cmp_cuda.cu:2255-2560). */
 int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out,
                            int B, int H, int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream);
+
+/* cats_mlp(y_out mode) for callers that cannot allocate device memory or carry a workspace -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose ops
+ * cudaMalloc per call).  The scratch of the single-pass kernels (per-workgroup partial sums and counts, 8 MiB + 4 KiB)
+ * lives in a device array inside the library, one copy per GPU, held until the process ends; nothing is allocated or
+ * freed by the call.  Limits: 1..2 rows, B * H <= 8192, rows of at most 2048 16-byte vectors; anything else returns
+ * CATS_ERR_SCRATCH.  Same kernels and summation order as cats_mlp, so the same bits.  All calls on one GPU share
+ * that GPU's array: calls that overlap in time on one GPU (different streams, or a graph replay next to an eager
+ * call) race; calls on one stream, or otherwise ordered, are fine.  Nothing in the array has to be cleared between
+ * calls (every call overwrites what it reads). */
+int cats_mlp_noalloc(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out,
+                     int B, int H, int I, int dtype, float threshold, void* stream);
 
 /* One launch of cats_mlp(y_out mode) alone, for per-kernel timing and profiling: stage 1 = the streaming launch (gate, up
  * and, for 1..2 rows, down into per-workgroup partial sums), stage 2 = the launch that finishes y from what stage 1 left in
