@@ -182,9 +182,7 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   d.flags = flags;
   d.y32 = y32;
   d.y_out = y_out;
-  d.residual = residual;
   d.partial = (float*)(ws + l.partial);
-  d.done = (uint32_t*)(ws + l.counters);
   d.count_out = count_out;
   d.H = H; d.I = I; d.nb = B;
   d.row_vecs = H / vec_elems(dtype);
@@ -209,6 +207,21 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   if (dtype == CATS_F16) e = launch_down<F16>(bt, zf32, d, block, s);
   else if (dtype == CATS_BF16) e = launch_down<BF16>(bt, zf32, d, block, s);
   else e = launch_down<F32>(bt, zf32, d, block, s);
+  if (e != hipSuccess) return CATS_ERR_LAUNCH;
+  if (y_out == nullptr) return CATS_OK;
+  // y_out mode: the groups' partial sums are added, rounded (and the residual added) by the reduction launch
+  ReduceArgs r;
+  memset(&r, 0, sizeof(r));
+  r.partial = d.partial;
+  r.y_out = y_out;
+  r.residual = residual;
+  r.G = d.ngroup;
+  r.BH = B * H;
+  FusedArgs none;
+  memset(&none, 0, sizeof(none));
+  if (dtype == CATS_F16) e = launch_fused<F16>(1, 0, 2, none, r, s);
+  else if (dtype == CATS_BF16) e = launch_fused<BF16>(1, 0, 2, none, r, s);
+  else e = launch_fused<F32>(1, 0, 2, none, r, s);
   return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
 }
 

@@ -5,10 +5,11 @@
 // active row in its range: the waves deal the active rows round-robin and keep up to U loads in flight per
 // lane.  Partial sums stay in registers (VEC per lane per batch row) and are folded across the waves of the
 // workgroup through LDS.  Across workgroups there are two ways out:
-//   * y_out (dtype output): every workgroup stores its slab partial to scratch, the last workgroup of the slab
-//     to finish adds the ngroup partials in group order and writes the rounded result.  No atomics on data
-//     (32 workgroups adding into the same 16 cache lines serialise for microseconds), a fixed summation order
-//     (bitwise reproducible output), nothing to zero between calls.
+//   * y_out (dtype output): every workgroup stores its partial sums to scratch, [group][b][H]; the reduction launch
+//     that follows (reduce_partials_kernel) adds the ngroup partials in group order and writes the rounded result.
+//     No atomics on data (32 workgroups adding into the same 16 cache lines serialise for microseconds), a fixed
+//     summation order (bitwise reproducible output), nothing to zero between calls, no synchronisation between
+//     workgroups other than the launch boundary.
 //   * y32 (caller's fp32 accumulator, "atomic_gemv" semantics): one fp32 atomic per column per workgroup.
 // blockIdx % nslab picks the slab, so with 8 slabs every XCD (workgroups are dealt round-robin over the 8
 // XCDs) streams one slab.
@@ -30,9 +31,7 @@ struct DownArgs {
   const uint8_t* flags;   // alternative to mask: (nb, I) flag bytes, OR-ed over the batch on the fly; NULL = use mask
   float* y32;             // (nb, H) the caller's fp32 accumulator (atomics), used when y_out == NULL
   void* y_out;            // (nb, H) dtype
-  const void* residual;   // optional (nb, H) dtype, y_out mode: y = residual + round(sum); may alias y_out
-  float* partial;         // y_out mode: [nslab][ngroup][B][64*VEC] fp32 slab partials
-  uint32_t* done;         // y_out mode: per-slab arrival counters, zero between calls
+  float* partial;         // y_out mode: [ngroup][nb][H] fp32 partial sums, finished by reduce_partials_kernel
   int32_t* count_out;     // optional: number of active neurons
   int H, I, nb;
   int row_vecs;           // H / VEC
@@ -92,7 +91,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   constexpr int kSlabCols = kWave * VEC;
   constexpr int UP = U / 2;  // row pairs in flight per lane
   constexpr bool kPacked = sizeof(st) == 2;  // 16-bit types: z of a row pair travels as one packed dword
-  extern __shared__ float s_dyn[];
+  extern __shared__ __attribute__((aligned(16))) float s_dyn[];  // 8- and 16-byte LDS accesses below: a 4-byte-aligned base makes every one of them a slow unaligned access
   // dynamic LDS, streaming phase: [chunk] int list | [B][chunk] z in storage type (indexed by j - j0)
   //                               | 16-bit types: [chunk / 2][B] packed z pairs in list order
   // afterwards reused for the fold: [nwaves / 2][B][VEC][64] float
@@ -101,7 +100,6 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   uint32_t* s_zp = (uint32_t*)(s_dyn + p.chunk) + (B * p.chunk * sizeof(st) + 3) / 4;
   float* s_red = s_dyn;
   __shared__ int s_n;
-  __shared__ int s_last;
 
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -213,73 +211,52 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
 
   CATS_STAMP(2);
   // ---- 3. fold the waves through LDS -----------------------------------------------------------------------
-  // Up to four batch rows (16 waves x 4 x 2 KiB = 128 KiB of LDS): every wave writes its sums, one barrier, one thread per column adds the waves in wave
-  // order and stores the slab partial.  More batch rows would not fit in LDS that way: pairwise rounds instead
-  // (upper half writes, lower half adds), after which wave 0 holds the partial.
-  // Partial layout (both ways): float (b, pair p, lane l, k) at b*kSlabCols + p*128 + l*2 + k  is column
-  // (slab*64 + l) * VEC + 2p + k.
-  float* mypart = p.partial + ((size_t)slab * p.ngroup + group) * B * kSlabCols;
+  // Up to four batch rows at a time (16 waves x 4 x 2 KiB = 128 KiB of LDS): every wave writes its sums, one barrier,
+  // one thread per column adds the waves in wave order.  Eight batch rows take two such passes.  LDS layout of a pass:
+  // float (wave w, row b, pair q, lane l, k) at ((w * FB + b) * VEC/2 + q) * 128 + l * 2 + k  is column
+  // (slab * 64 + l) * VEC + 2 q + k  -- lanes write float2, consecutive lanes consecutive banks.
+  // y_out mode: the folded sums go to the scratch partial [group][b][H]; the reduction launch that follows adds the
+  // groups in order (a fixed summation order: bitwise reproducible output, nothing to zero between calls, no
+  // cross-workgroup synchronisation inside this kernel).  y32 mode (the caller's fp32 accumulator, "atomic_gemv"
+  // semantics): one fp32 atomic per column per workgroup.
+  constexpr int FB = B < 4 ? B : 4;  // batch rows folded per pass
   __syncthreads();  // the list and z are dead from here on; their LDS is reused
-  if constexpr (B <= 4) {
-    {
-      float* dst = s_red + (size_t)wave * B * kSlabCols + lane * 2;
 #pragma unroll
-      for (int b = 0; b < B; b++)
+  for (int b0 = 0; b0 < B; b0 += FB) {
+    if (b0 > 0) __syncthreads();  // the previous pass has been read
+    {
+      float* dst = s_red + (size_t)wave * FB * kSlabCols + lane * 2;
+#pragma unroll
+      for (int b = 0; b < FB; b++)
 #pragma unroll
         for (int e = 0; e < VEC; e += 2) {
-          float2 v2 = {acc[b][e], acc[b][e + 1]};
+          float2 v2 = {acc[b0 + b][e], acc[b0 + b][e + 1]};
           *(float2*)(dst + b * kSlabCols + (e >> 1) * (2 * kWave)) = v2;
         }
     }
     __syncthreads();
-    for (int f = tid; f < p.nb * kSlabCols; f += blockDim.x) {
-      float s = 0.f;
-      for (int w = 0; w < nwaves; w++) s += s_red[(size_t)w * B * kSlabCols + f];
-      if (p.y_out) {
-        __hip_atomic_store(&mypart[f], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      } else {
-        const int b = f / kSlabCols, c = f - b * kSlabCols;
-        const int col = (slab * kWave + ((c & (2 * kWave - 1)) >> 1)) * VEC + (c / (2 * kWave)) * 2 + (c & 1);
-        if (col < p.H && n > 0) unsafeAtomicAdd(&p.y32[(size_t)b * p.H + col], s);
+    const int rows = min(FB, p.nb - b0);  // live batch rows of this pass (may be <= 0)
+    // One item = four consecutive columns of one batch row: two float2 per wave from LDS, one 16-byte store.  Whole
+    // sectors are written (a store of part of a 32-byte sector makes the memory side read the sector first).
+    constexpr int kQuads = kSlabCols / 4;
+    for (int it = tid; it < rows * kQuads; it += blockDim.x) {
+      const int b = it / kQuads, r = it - b * kQuads;
+      const int l = r / (VEC / 4), h = r - l * (VEC / 4);  // lane that owned the columns, which quarter of its VEC
+      const float* src = s_red + b * kSlabCols + (2 * h) * (2 * kWave) + l * 2;
+      float4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+      for (int w = 0; w < nwaves; w++) {
+        const float2 lo = *(const float2*)(src + (size_t)w * FB * kSlabCols);
+        const float2 hi = *(const float2*)(src + (size_t)w * FB * kSlabCols + 2 * kWave);
+        s4.x += lo.x; s4.y += lo.y; s4.z += hi.x; s4.w += hi.y;
       }
-    }
-  } else {
-    for (int half = nwaves >> 1; half >= 1; half >>= 1) {
-      if (wave >= half && wave < 2 * half) {
-        float* dst = s_red + (size_t)(wave - half) * B * kSlabCols;
-#pragma unroll
-        for (int b = 0; b < B; b++)
-#pragma unroll
-          for (int e = 0; e < VEC; e++) dst[(b * VEC + e) * kWave + lane] = acc[b][e];
-      }
-      __syncthreads();
-      if (wave < half) {
-        const float* src = s_red + (size_t)wave * B * kSlabCols;
-#pragma unroll
-        for (int b = 0; b < B; b++)
-#pragma unroll
-          for (int e = 0; e < VEC; e++) acc[b][e] += src[(b * VEC + e) * kWave + lane];
-      }
-      __syncthreads();
-    }
-    if (wave == 0) {
-#pragma unroll
-      for (int b = 0; b < B; b++) {
-        if (b < p.nb) {  // uniform
-          if (p.y_out) {
-#pragma unroll
-            for (int e = 0; e < VEC; e += 2) {
-              const uint64_t two = (uint64_t)__float_as_uint(acc[b][e]) | ((uint64_t)__float_as_uint(acc[b][e + 1]) << 32);
-              __hip_atomic_store((uint64_t*)&mypart[b * kSlabCols + (e >> 1) * (2 * kWave) + 2 * lane], two, __ATOMIC_RELAXED,
-                                 __HIP_MEMORY_SCOPE_AGENT);
-            }
-          } else {
-#pragma unroll
-            for (int e = 0; e < VEC; e++) {
-              const int col = (slab * kWave + lane) * VEC + e;
-              if (col < p.H && n > 0) unsafeAtomicAdd(&p.y32[(size_t)b * p.H + col], acc[b][e]);
-            }
-          }
+      const int col = (slab * kWave + l) * VEC + 4 * h;
+      if (col < p.H) {  // H is a multiple of VEC, so a quad is inside or outside as a whole
+        if (p.y_out) {
+          *(float4*)&p.partial[((size_t)group * p.nb + b0 + b) * p.H + col] = s4;
+        } else if (n > 0) {
+          float* y = &p.y32[(size_t)(b0 + b) * p.H + col];
+          unsafeAtomicAdd(y, s4.x); unsafeAtomicAdd(y + 1, s4.y); unsafeAtomicAdd(y + 2, s4.z); unsafeAtomicAdd(y + 3, s4.w);
         }
       }
     }
@@ -302,65 +279,8 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
       for (int w = 0; w < nwaves; w++) tot += s_red[w];
       *p.count_out = (int)tot;
     }
-    __syncthreads();
   }
   CATS_STAMP(3);
-  if (p.y_out == nullptr) return;
-
-  // ---- 4. last workgroup of the slab adds the partials in group order and writes y ---------------------------
-  // Ordering without a release / acquire fence pair (at agent scope those write back and invalidate the whole
-  // L2 of the XCD, which costs far more than this kernel): partials are written and read with agent-scope
-  // atomic stores / loads, which are coherent across the device by themselves.  Every wave waits until its own
-  // stores have been acknowledged (s_waitcnt vmcnt(0)), the barrier joins them, and only then is the slab counter bumped -- so when a
-  // workgroup reads "I am last" every partial of the slab is in place, and the loads below, issued after
-  // that read, see them.
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), expcnt / lgkmcnt untouched: this wave's partial stores are acknowledged
-  __syncthreads();                     // ... and so are everybody else's
-  CATS_STAMP(4);
-  if (tid == 0) {
-    const uint32_t prev = __hip_atomic_fetch_add(&p.done[slab], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    s_last = prev == (uint32_t)p.ngroup - 1u;
-  }
-  __syncthreads();
-  CATS_STAMP(5);
-  if (!s_last) return;
-  const uint64_t* slabpart = (const uint64_t*)(p.partial + (size_t)slab * p.ngroup * B * kSlabCols);
-  constexpr int kPairs = VEC / 2 * kWave;  // 64-bit items per batch row and group
-  constexpr int kInFlight = 32;  // with the default 32 groups every partial of an item is requested in one go
-  for (int item = tid; item < p.nb * kPairs; item += blockDim.x) {
-    const int b = item / kPairs, r = item - b * kPairs;
-    const int e = (r >> 6) * 2, l = r & 63;
-    const int col = (slab * kWave + l) * VEC + e;
-    float s0 = 0.f, s1 = 0.f;
-    for (int g0 = 0; g0 < p.ngroup; g0 += kInFlight) {  // independent loads in flight, added in group order
-      uint64_t t[kInFlight];
-#pragma unroll
-      for (int u = 0; u < kInFlight; u++) {
-        const int gg = min(g0 + u, p.ngroup - 1);
-        t[u] = __hip_atomic_load(&slabpart[((size_t)gg * B + b) * kPairs + r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-#pragma unroll
-      for (int u = 0; u < kInFlight; u++) {
-        if (g0 + u < p.ngroup) {
-          s0 += __uint_as_float((uint32_t)t[u]);
-          s1 += __uint_as_float((uint32_t)(t[u] >> 32));
-        }
-      }
-    }
-    if (col < p.H) {
-      st* y = (st*)p.y_out + (size_t)b * p.H + col;
-      if (p.residual) {  // the MLP output is rounded to the storage type first, as a module returning a tensor would
-        const st* res = (const st*)p.residual + (size_t)b * p.H + col;
-        s0 = DT::rnd(s0) + DT::tof(res[0]);
-        s1 = DT::rnd(s1) + DT::tof(res[1]);
-      }
-      y[0] = DT::fromf(s0);
-      y[1] = DT::fromf(s1);
-    }
-  }
-  if (tid == 0) __hip_atomic_store(&p.done[slab], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __builtin_amdgcn_s_waitcnt(0x0F70);
-  CATS_STAMP(6);
 }
 
 }  // namespace cats

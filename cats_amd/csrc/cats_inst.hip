@@ -120,7 +120,7 @@ hipError_t launch_down_one(const DownArgs& a, int block, hipStream_t stream) {
   // (index list, z, and for 16-bit types the packed z pairs)
   const size_t zbytes = (size_t)B * a.chunk * sizeof(typename DT::st);
   const size_t lds_stream = (size_t)a.chunk * sizeof(int) + (zbytes + 3) / 4 * 4 + (sizeof(typename DT::st) == 2 ? zbytes + 4 * B : 0);
-  const size_t lds_fold = (size_t)(B <= 4 ? nwaves : nwaves / 2) * B * kWave * DT::VEC * sizeof(float);
+  const size_t lds_fold = (size_t)nwaves * (B < 4 ? B : 4) * kWave * DT::VEC * sizeof(float);  // up to four batch rows per pass
   const size_t lds = (lds_stream > lds_fold ? lds_stream : lds_fold) + 64;
   if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3(a.nslab * a.ngroup), dim3(block), lds, stream, a);
