@@ -86,6 +86,7 @@ def main():
     ap.add_argument("--extra", default="mistral,batch,70b,entry",
                     help="which of the other measurements to run: mistral (bf16, heavy-tailed), batch (2/4/8), 70b (8192->28672), "
                          "entry (each drop-in entry point alone)")
+    ap.add_argument("--entries", default="", help="with --extra entry: comma-separated entry points to time (default: all)")
     ap.add_argument("--no-graph", action="store_true", help="time plain stream launches only")
     ap.add_argument("--decode", action="store_true", help="(default) run the 32-layer decode loop (config 5)")
     ap.add_argument("--no-decode", action="store_true", help="skip the 32-layer decode loop")
@@ -330,7 +331,8 @@ def main():
         out["other_configs"] = other_configs(torch, F, capi, L, max(200, args.steps // 4), max(50, args.warmup // 4), extra)
 
     if "entry" in extra:
-        out["entry_points"] = entry_points(torch, F, capi, max(200, args.steps // 4), max(50, args.warmup // 4))
+        out["entry_points"] = entry_points(torch, F, capi, max(200, args.steps // 4), max(50, args.warmup // 4),
+                                           {e.strip() for e in args.entries.split(",") if e.strip()})
 
     if not args.no_decode:
         from cats_amd import decoder
@@ -425,7 +427,7 @@ def other_configs(torch, F, capi, L, steps, warmup, which):
     return res
 
 
-def entry_points(torch, F, capi, steps, warmup):
+def entry_points(torch, F, capi, steps, warmup, only=()):
     """Latency of each drop-in entry point alone on the headline layer (Llama shape, fp16, batch 1, 50 % sparsity),
     with the algorithmic bytes it has to move.  Weight sets rotate as in the headline run."""
     dev = torch.device("cuda:0")
@@ -446,6 +448,11 @@ def entry_points(torch, F, capi, steps, warmup):
     for st in sets:
         st["a"], st["flag"] = capi.gate_flag(x, st["wg"], t)
         st["z"] = capi.up_flag(x, st["wu"], st["a"], st["flag"])
+        # the same active set as a sorted index list with compact activations / intermediates (the DejaVu-style interface)
+        st["idx"] = torch.nonzero(st["flag"][0]).flatten()
+        st["a_c"] = st["a"][0][st["idx"]].contiguous()
+        st["z_c"] = st["z"][:, st["idx"]].contiguous()
+        st["wg_t"] = st["wg"].t().contiguous()
     k = sum(int(st["flag"].sum()) for st in sets) / nsets
     nw = torch.ones(H, dtype=torch.float16, device=dev)
     # fuse_gemv_cmp: device part only (the reference's op also copies the count to the host, which is a stream sync)
@@ -453,6 +460,8 @@ def entry_points(torch, F, capi, steps, warmup):
     idx = torch.empty(I, dtype=torch.int64, device=dev)
     cnt = torch.zeros(1, dtype=torch.int32, device=dev)
     L = capi.lib()
+    import flash_gemv as fg
+
     pv = lambda t_: ctypes.c_void_p(t_.data_ptr())
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -478,6 +487,12 @@ def entry_points(torch, F, capi, steps, warmup):
         ("cats_gate_compact", "fuse_gemv_cmp (ordered index list + count, device part)", full, compact),
         ("cats_up_flag", "fuse_flag_gemv_local, gather_gemv_elemul_flag_3d", act_rows, lambda st: capi.up_flag(x, st["wu"], st["a"], st["flag"])),
         ("cats_down_flag", "atomic_gemv, gather_transposed_gemv_flag_3d", act_rows, lambda st: capi.down_flag(st["z"], st["wdt"], st["flag"], ws)),
+        ("cats_up_index", "gather_gemv, gather_gemv_elemul_indirect_index_2d (sorted index list)", act_rows,
+         lambda st: capi.up_index(x, st["wu"], st["idx"], None, st["a_c"])),
+        ("cats_down_index", "gather_transposed_gemv, gather_transposed_gemv_indirect_index_2d (sorted index list)", act_rows,
+         lambda st: capi.down_index(st["z_c"], st["wdt"], st["idx"], ws)),
+        ("flash_gemv.flag_gemv_gemv_dejavu", "the reference's index-list composite: torch gate GEMV + SiLU + nonzero (host sync), index-list up and down",
+         full + 2 * act_rows, lambda st: fg.flag_gemv_gemv_dejavu(x, st["wg_t"], st["wu"], st["wdt"], t)),
         ("cats_up_down", "gemv_gemv_triton (gate activations given)", 2 * act_rows, lambda st: capi.up_down(x, st["a"], st["wu"], st["wdt"], t, ws)),
         ("cats_gate_up", "fuse_gemv_flag_gemv", full + act_rows, lambda st: capi.gate_up(x, st["wg"], st["wu"], t)),
         ("cats_mlp", "flag_gemv_gemv_atomic, fuse_gemv_flag_gemv_gemv", full + 2 * act_rows, lambda st: capi.mlp(x, st["wg"], st["wu"], st["wdt"], t, ws)),
@@ -487,6 +502,8 @@ def entry_points(torch, F, capi, steps, warmup):
     ]
     res = []
     for name, replaces, nbytes, fn in table:
+        if only and name not in only:
+            continue
         us = timed(fn)
         res.append(dict(entry_point=name, replaces=replaces, us=round(us, 2), weight_MB=round(nbytes / 1e6, 1),
                         GBps=round(nbytes / us * 1e-3, 1), hbm_frac=round(nbytes / us * 1e-3 / HBM_PEAK_GBPS, 4)))

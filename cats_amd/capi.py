@@ -22,7 +22,7 @@ DTYPE_CODE = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
 SYMBOLS = (
     "cats_version", "cats_status_string", "cats_workspace_bytes", "cats_workspace_init", "cats_gate_flag",
     "cats_gate_compact", "cats_read_count", "cats_up_flag", "cats_down_flag", "cats_gate_up", "cats_mlp",
-    "cats_mlp_rowmajor_down", "cats_mlp_norm_residual", "cats_up_down", "cats_set_tuning", "cats_mlp_stage", "cats_mlp_noalloc",
+    "cats_mlp_rowmajor_down", "cats_mlp_norm_residual", "cats_up_down", "cats_set_tuning", "cats_mlp_stage", "cats_mlp_noalloc", "cats_up_index", "cats_down_index",
 )
 
 
@@ -54,6 +54,8 @@ def lib() -> ctypes.CDLL:
         L.cats_up_down.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_up_down.restype = i32
         L.cats_mlp_stage.argtypes = [i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_mlp_stage.restype = i32
         L.cats_mlp_noalloc.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp]; L.cats_mlp_noalloc.restype = i32
+        L.cats_up_index.argtypes = [vp, vp, vp, i32, vp, vp, i32, vp, i32, i32, i32, i32, vp]; L.cats_up_index.restype = i32
+        L.cats_down_index.argtypes = [vp, vp, vp, i32, vp, vp, i32, i32, i32, i32, vp, sz, vp]; L.cats_down_index.restype = i32
         L.cats_set_tuning.argtypes = [i32, i32, i32, i32]; L.cats_set_tuning.restype = i32
         _lib = L
     return _lib
@@ -155,6 +157,30 @@ def mlp(x, wgate, wup, wdown_t, threshold, ws: Workspace, y=None, want_flag=Fals
     if want_flag or want_count:
         return out, flag, count
     return out
+
+
+ACTIVATIONS = {"id": 0, "relu": 1, "squared_relu": 2, "swish": 3}
+
+
+def up_index(x, w, idx, bias=None, scale=None, activation="id"):
+    """out[b, m] = scale[m] * act(x[b] . w[idx[m]] + bias[idx[m]]); idx int64 (M,).  Returns (B, M) in x.dtype."""
+    B, H, Z = _dims(x, w)
+    M = int(idx.numel())
+    out = torch.empty(B, M, dtype=x.dtype, device=x.device)
+    check(lib().cats_up_index(_p(x), _p(w), _p(idx), M, _p(bias), _p(scale), ACTIVATIONS[activation], _p(out), B, H, Z,
+                              DTYPE_CODE[x.dtype], _stream(x)), "cats_up_index")
+    return out
+
+
+def down_index(z, wdown_t, idx, ws: Workspace, bias=None):
+    """y[b] = sum_m z[b, m] * wdown_t[idx[m]] (+ bias); z (B, M) aligned with idx.  Returns (B, H) in z.dtype."""
+    Z, H = wdown_t.shape
+    M = int(idx.numel())
+    B = z.shape[0]
+    y = torch.empty(B, H, dtype=z.dtype, device=z.device)
+    check(lib().cats_down_index(_p(z), _p(wdown_t), _p(idx), M, _p(bias), _p(y), B, H, Z, DTYPE_CODE[z.dtype], _p(ws.buf), ws.nbytes,
+                                _stream(z)), "cats_down_index")
+    return y
 
 
 def mlp_noalloc(x, wgate, wup, wdown_t, threshold, y):

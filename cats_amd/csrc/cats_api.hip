@@ -173,13 +173,16 @@ int do_rows(int mode, int dtype, const RowsArgs& a_in, hipStream_t s) {
 
 // Sparse down over mask words already in the workspace.
 int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_out, int32_t* count_out, int B, int H, int I,
-            int dtype, char* ws, const WsLayout& l, hipStream_t s, const void* residual = nullptr, const uint8_t* flags = nullptr) {
+            int dtype, char* ws, const WsLayout& l, hipStream_t s, const void* residual = nullptr, const uint8_t* flags = nullptr,
+            const int64_t* idx = nullptr, int M = 0, const void* bias = nullptr) {
   DownArgs d;
   memset(&d, 0, sizeof(d));
   d.wd = (const u32x4*)wdown_t;
   d.z = z;
   d.mask = (const uint8_t*)(ws + l.mask);
   d.flags = flags;
+  d.idx = idx;
+  d.M = M;
   d.y32 = y32;
   d.y_out = y_out;
   d.partial = (float*)(ws + l.partial);
@@ -197,9 +200,10 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   int ngroup = g_tuning.down_groups > 0 ? g_tuning.down_groups : 256 / d.nslab;
   if (ngroup < 1) ngroup = 1;
   if (ngroup > kMaxGroups) ngroup = kMaxGroups;
-  d.chunk = ((I + ngroup - 1) / ngroup + 7) / 8 * 8;
+  const int zcols = idx ? M : I;  // what the groups split: the index list, or the neuron range
+  d.chunk = ((zcols + ngroup - 1) / ngroup + 7) / 8 * 8;
   if ((size_t)d.chunk * (1 + bt) * 4 > 96 * 1024) return CATS_ERR_SHAPE;  // a group's list and z must fit in LDS
-  d.ngroup = (I + d.chunk - 1) / d.chunk;
+  d.ngroup = (zcols + d.chunk - 1) / d.chunk;
 #ifdef CATS_TIMING
   d.tbuf = g_tbuf_down;
 #endif
@@ -215,6 +219,8 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   r.partial = d.partial;
   r.y_out = y_out;
   r.residual = residual;
+  r.bias = bias;
+  r.H = H;
   r.G = d.ngroup;
   r.BH = B * H;
   FusedArgs none;
@@ -279,6 +285,7 @@ int do_fused(FusedArgs& f, int grid, int stage, void* y_out, const void* residua
   r.y_out = y_out;
   r.residual = residual;
   r.count_out = count_out;
+  r.H = f.H;
   r.G = grid;
   r.BH = f.nb * f.H;
   const int bt = batch_template(f.nb);
@@ -402,17 +409,30 @@ int cats_gate_compact(const void* x, const void* wgate, void* vals_out, int64_t*
   WsLayout l;
   st = check_ws(ws, ws_bytes, H, I, l);
   if (st) return st;
+  // launch 1: the gate pass, activations and mask bytes into the workspace
   RowsArgs a;
   fill_rows(a, x, wgate, H, I, 1, dtype);
   a.a_out = (char*)ws + l.atmp;
   a.mask_out = (uint8_t*)ws + l.mask;
-  a.arrive = (uint32_t*)((char*)ws + l.counters + 512);
-  a.arrive_sub = (uint32_t*)((char*)ws + l.counters + 1024);
-  a.idx_out = idx_out;
-  a.vals_out = vals_out;
-  a.count_out = count_out;
   a.t = round_through(dtype, threshold);
-  return do_rows(kGate, dtype, a, (hipStream_t)stream);
+  st = do_rows(kGate, dtype, a, (hipStream_t)stream);
+  if (st) return st;
+  // launch 2: mask bytes -> ascending list, values, count
+  CompactArgs c;
+  c.mask = a.mask_out;
+  c.a = a.a_out;
+  c.idx_out = idx_out;
+  c.vals_out = vals_out;
+  c.count_out = count_out;
+  c.N = I;
+  const int nbytes = (I + 7) / 8;
+  int groups = (nbytes + 255) / 256;  // at least one pass of 256 bytes each; more groups than that gain nothing
+  if (groups > 64) groups = 64;
+  c.bytes_per_group = (nbytes + groups - 1) / groups;
+  groups = (nbytes + c.bytes_per_group - 1) / c.bytes_per_group;  // the last group's range is never empty: it writes the count
+  if (elem_size(dtype) == 2) hipLaunchKernelGGL(compact_kernel<2>, dim3(groups), dim3(256), 0, (hipStream_t)stream, c);
+  else hipLaunchKernelGGL(compact_kernel<4>, dim3(groups), dim3(256), 0, (hipStream_t)stream, c);
+  return hipGetLastError() == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
 }
 
 int cats_read_count(const int32_t* count_dev, void* stream) {
@@ -653,6 +673,56 @@ int cats_mlp_stage(int stage, const void* x, const void* wgate, const void* wup,
   return mlp_pass(x, wgate, wup, wdown_t, y_out, nullptr, nullptr, nullptr, B, H, I, dtype, threshold, ws, ws_bytes, stream, stage);
 }
 
+int cats_up_index(const void* x, const void* w, const int64_t* idx, int M, const void* bias, const void* scale, int activation,
+                  void* out, int B, int H, int Z, int dtype, void* stream) {
+  if (M == 0) return (B >= 1 && B <= kKernelBatch) ? CATS_OK : CATS_ERR_BATCH;
+  int st = check_common(B, H, Z, dtype);
+  if (st) return st;
+  if (M < 0 || activation < 0 || activation > 3) return CATS_ERR_SHAPE;
+  if (!x || !w || !idx || !out) return CATS_ERR_NULL;
+  if (!aligned16(x) || !aligned16(w)) return CATS_ERR_ALIGN;
+  RowsArgs a;
+  fill_rows(a, x, w, H, M, B, dtype);
+  a.row_idx = idx;
+  a.w_rows = Z;
+  a.bias = bias;
+  a.scale = scale;
+  a.activation = activation;
+  a.zt_out = out;
+  return do_rows(kUpIndex, dtype, a, (hipStream_t)stream);
+}
+
+int cats_down_index(const void* z, const void* wdown_t, const int64_t* idx, int M, const void* bias, void* y_out, int B, int H, int Z,
+                    int dtype, void* ws, size_t ws_bytes, void* stream) {
+  int st = check_common(B, H, Z, dtype);
+  if (st) return st;
+  if (M < 0) return CATS_ERR_SHAPE;
+  if (!wdown_t || !y_out || (M > 0 && (!z || !idx))) return CATS_ERR_NULL;
+  if (!aligned16(wdown_t)) return CATS_ERR_ALIGN;
+  WsLayout l;
+  st = check_ws(ws, ws_bytes, H, Z, l);
+  if (st) return st;
+  if (M == 0) {
+    // an empty list: y = bias or 0, written by the reduction over zero partials
+    ReduceArgs r;
+    memset(&r, 0, sizeof(r));
+    r.partial = (float*)((char*)ws + l.partial);
+    r.y_out = y_out;
+    r.bias = bias;
+    r.H = H;
+    r.G = 0;
+    r.BH = B * H;
+    FusedArgs none;
+    memset(&none, 0, sizeof(none));
+    hipError_t e;
+    if (dtype == CATS_F16) e = launch_fused<F16>(1, 0, 2, none, r, (hipStream_t)stream);
+    else if (dtype == CATS_BF16) e = launch_fused<BF16>(1, 0, 2, none, r, (hipStream_t)stream);
+    else e = launch_fused<F32>(1, 0, 2, none, r, (hipStream_t)stream);
+    return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+  }
+  return do_down(z, false, wdown_t, nullptr, y_out, nullptr, B, H, Z, dtype, (char*)ws, l, (hipStream_t)stream, nullptr, nullptr, idx, M, bias);
+}
+
 int cats_mlp_noalloc(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,
                      int dtype, float threshold, void* stream) {
   int st = check_common(B, H, I, dtype);
@@ -683,6 +753,7 @@ int cats_mlp_noalloc(const void* x, const void* wgate, const void* wup, const vo
   r.partial = f.partial;
   r.counts = f.counts;
   r.y_out = y_out;
+  r.H = H;
   r.G = grid;
   r.BH = B * H;
   const int bt = batch_template(B);

@@ -29,6 +29,8 @@ struct DownArgs {
   const void* z;          // (nb, I) fp32 or dtype
   const uint8_t* mask;    // ceil(I/8) bytes, bit j = neuron j active for some batch row
   const uint8_t* flags;   // alternative to mask: (nb, I) flag bytes, OR-ed over the batch on the fly; NULL = use mask
+  const int64_t* idx;     // alternative to both: an index list of M weight rows (any order, duplicates add up, entries outside
+  int M;                  //   [0, I) contribute nothing); z is then (nb, M), aligned with the list, and the groups split the list
   float* y32;             // (nb, H) the caller's fp32 accumulator (atomics), used when y_out == NULL
   void* y_out;            // (nb, H) dtype
   float* partial;         // y_out mode: [ngroup][nb][H] fp32 partial sums, finished by reduce_partials_kernel
@@ -107,12 +109,21 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   const int nwaves = blockDim.x >> 6;                         // a power of two
   const int slab = blockIdx.x % p.nslab;
   const int group = blockIdx.x / p.nslab;
-  const int j0 = group * p.chunk;
-  const int j1 = min(j0 + p.chunk, p.I);
+  const bool by_list = p.idx != nullptr;          // uniform
+  const int zcols = by_list ? p.M : p.I;          // row length of z
+  const int j0 = group * p.chunk;                 // first neuron (or list position) of this group
+  const int j1 = min(j0 + p.chunk, zcols);
   CATS_STAMP(0);
 
   // ---- 1. wave 0: mask bytes of the range -> ascending index list; the other waves: z of the range -> LDS ----
-  if (wave == 0) {
+  if (wave == 0 && by_list) {
+    // the list is given: entry i of the range is weight row idx[j0 + i]
+    for (int i = lane; i < j1 - j0; i += kWave) {
+      const long long j = p.idx[j0 + i];
+      s_list[i] = (j >= 0 && j < (long long)p.I) ? (int)j : 0;  // an entry outside the matrix reads row 0 against z = 0
+    }
+    if (lane == 0) s_n = max(j1 - j0, 0);
+  } else if (wave == 0) {
     int base = 0;
     for (int byte0 = j0 >> 3; byte0 * 8 < j1; byte0 += kWave) {
       const int byte = byte0 + lane;
@@ -148,8 +159,13 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
     const int total = p.nb * span;
     for (int i = tid - kWave; i < total; i += blockDim.x - kWave) {
       const int b = i / span, q = i - b * span;
-      const size_t o = (size_t)b * p.I + j0 + q;
-      s_z[b * p.chunk + q] = ZF32 ? DT::fromf(((const float*)p.z)[o]) : ((const st*)p.z)[o];
+      const size_t o = (size_t)b * zcols + j0 + q;
+      st zv = ZF32 ? DT::fromf(((const float*)p.z)[o]) : ((const st*)p.z)[o];
+      if (by_list) {
+        const long long j = p.idx[j0 + q];
+        if (!(j >= 0 && j < (long long)p.I)) zv = DT::fromf(0.f);
+      }
+      s_z[b * p.chunk + q] = zv;
     }
     for (int i = p.nb * p.chunk + tid - kWave; i < B * p.chunk; i += blockDim.x - kWave) s_z[i] = DT::fromf(0.f);
   }
@@ -159,7 +175,9 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   if (kPacked) {
     for (int i = tid; i < nfull * B; i += blockDim.x) {
       const int k = i / B, b = i - k * B;
-      const uint32_t za = s_z[b * p.chunk + s_list[2 * k] - j0], zb = s_z[b * p.chunk + s_list[2 * k + 1] - j0];
+      // z of a list entry sits at its neuron's offset in the range, or (index-list mode) at its position in the list
+      const uint32_t za = s_z[b * p.chunk + (by_list ? 2 * k : s_list[2 * k] - j0)];
+      const uint32_t zb = s_z[b * p.chunk + (by_list ? 2 * k + 1 : s_list[2 * k + 1] - j0)];
       s_zp[i] = za | (zb << 16);
     }
     __syncthreads();
@@ -198,7 +216,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
     for (int u = 0; u < UP; u++) {
       if (u < cnt) {
         if constexpr (kPacked) PairAxpy16<DT, B>::run(wa[u], wb[u], s_zp + kk[u] * B, acc);
-        else PairAxpy<DT, B>::run(wa[u], wb[u], s_z + (ja[u] - j0), s_z + (jb[u] - j0), p.chunk, acc);
+        else PairAxpy<DT, B>::run(wa[u], wb[u], s_z + (by_list ? 2 * kk[u] : ja[u] - j0), s_z + (by_list ? 2 * kk[u] + 1 : jb[u] - j0), p.chunk, acc);
       }
     }
   }
@@ -206,7 +224,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
     const int j = __builtin_amdgcn_readfirstlane(s_list[n - 1]);
     const u32x4 w = load_stream(p.wd + (size_t)j * p.row_vecs + v);
 #pragma unroll
-    for (int b = 0; b < B; b++) DT::axpy(w, DT::tof(s_z[b * p.chunk + j - j0]), acc[b]);
+    for (int b = 0; b < B; b++) DT::axpy(w, DT::tof(s_z[b * p.chunk + (by_list ? n - 1 : j - j0)]), acc[b]);
   }
 
   CATS_STAMP(2);

@@ -61,6 +61,8 @@ struct ReduceArgs {
   const int32_t* counts; // [G]
   void* y_out;           // (nb, H) dtype, flattened to BH
   const void* residual;  // optional (nb, H) dtype; may alias y_out
+  const void* bias;      // optional (H,) dtype, added in fp32 before the rounding
+  int H;                 // row length of y (for the bias)
   int32_t* count_out;    // optional
   int G;                 // number of partials
   int BH;                // nb * H
@@ -447,6 +449,7 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(ReduceArgs p) {
       float tot = 0.f;
 #pragma unroll
       for (int l = 0; l < kReduceLanes; l++) tot += s_sum[l][tid];
+      if (p.bias) tot += DT::tof(((const st*)p.bias)[c % p.H]);
       if (p.residual) tot = DT::rnd(tot) + DT::tof(((const st*)p.residual)[c]);
       ((st*)p.y_out)[c] = DT::fromf(tot);
     }

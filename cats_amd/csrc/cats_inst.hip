@@ -88,7 +88,7 @@ hipError_t launch_rows_b(int mode, const RowsArgs& a, hipStream_t stream) {
   // measured on Llama-7B shapes: at 2 batch rows the wave-per-row kernel is still the faster one (28.4 vs 29.4 us)
   // The plain gate pass goes the same way (unless the caller wants the compact index list, which is a batch-1
   // feature), so a gate call and a fused call produce the same activations bit for bit.
-  if ((mode == kGateUp || (mode == kGate && a.idx_out == nullptr)) && B >= 4 && a.mma && MmaLaunch<DT>::supported(a))
+  if ((mode == kGateUp || mode == kGate) && B >= 4 && a.mma && MmaLaunch<DT>::supported(a))
     return MmaLaunch<DT>::run(a, mode == kGateUp, stream);
   const size_t lds = (size_t)B * ((a.nch + kCB - 1) / kCB * kCB) * kWave * sizeof(u32x4);
   const bool xlds = lds <= 128 * 1024;
@@ -108,6 +108,9 @@ hipError_t launch_rows_b(int mode, const RowsArgs& a, hipStream_t stream) {
     case kGemv:
       if (xlds) return launch_rows_one<DT, B, false, kGemv, true>(a, stream);
       return launch_rows_one<DT, B, false, kGemv, false>(a, stream);
+    case kUpIndex:
+      if (xlds) return launch_rows_one<DT, B, false, kUpIndex, true>(a, stream);
+      return launch_rows_one<DT, B, false, kUpIndex, false>(a, stream);
   }
   return hipErrorInvalidValue;
 }

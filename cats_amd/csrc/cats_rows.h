@@ -2,19 +2,22 @@
 // 128-bit streaming loads over the row, the dot products are accumulated in fp32 and folded across the
 // wave with DPP.  One template covers the four row-major passes of the CATS MLP:
 //
-//   kGate    a = SiLU(x . wgate[j]) ; flag = |a| > t ; optional mask words ; optional compact list
+//   kGate    a = SiLU(x . wgate[j]) ; flag = |a| > t ; optional mask bytes
 //   kGateUp  the gate pass, then for rows that came out active the matching wup row:  z = a * (x . wup[j])
 //   kUp      flags and a are given; fetch wup rows with any flag set:                  out = a * (x . wup[j])
 //   kGemv    plain y = W x (the dense (H,I) down projection over the zero-filled intermediate)
+//   kUpIndex an index list picks the weight rows:  out[b, m] = scale[m] * act(x[b] . w[idx[m]] + bias[idx[m]])
 //
 // x is staged once per workgroup in LDS, zero-padded to a whole number of 64-lane vectors, and read back
 // as one ds_read_b128 per lane per chunk (conflict-free: consecutive lanes, consecutive 16 bytes).
 #pragma once
+#include <type_traits>
+
 #include "cats_device.h"
 
 namespace cats {
 
-enum RowsMode { kGate = 0, kGateUp = 1, kUp = 2, kGemv = 3 };
+enum RowsMode { kGate = 0, kGateUp = 1, kUp = 2, kGemv = 3, kUpIndex = 4 };
 
 struct RowsArgs {
   const u32x4* x;        // (B, K) activations (K = row length of w)
@@ -27,12 +30,12 @@ struct RowsArgs {
   uint8_t* mask_out;     // kGate, kGateUp: ceil(N/8) bytes, bit j = OR over the batch of flag[b, j]; optional
   float* z32_out;        // kGateUp: (nb, N) fp32, written for rows fetched from wup only; kUp: fp32 out, all rows
   void* zt_out;          // kGateUp, kUp, kGemv: (nb, N) dtype, every row written (0 where inactive)
-  // compact list, kGate with nb == 1 only
-  uint32_t* arrive;      // zeroed counter; the last workgroup to finish builds the list and resets it
-  uint32_t* arrive_sub;  // 64 zeroed counters, 128 bytes apart: first level of the arrival count
-  int64_t* idx_out;
-  void* vals_out;
-  int32_t* count_out;
+  // index-list mode (kUpIndex): row m of the output is weight row row_idx[m]
+  const int64_t* row_idx;  // (N,) weight rows to fetch, any order, duplicates allowed; entries outside [0, w_rows) give 0
+  int w_rows;              // rows of w (bounds for row_idx)
+  const void* bias;        // optional (w_rows,) dtype, added to the dot product of weight row j as bias[j]
+  const void* scale;       // optional (N,) dtype, multiplies entry m after the activation (compact gate activations)
+  int activation;          // 0 id, 1 relu, 2 squared relu, 3 swish -- applied in fp32 before the one rounding
   int K;                 // row length in elements
   int N;                 // number of rows
   int nb;                // live batch rows (<= template B)
@@ -127,8 +130,6 @@ void rows_kernel(RowsArgs p) {
   typedef typename DT::st st;
   extern __shared__ u32x4 xs[];  // [B][round_up(nch, CB) * 64] vectors (XLDS only)
   __shared__ uint32_t s_maskbits;
-  __shared__ int s_last;
-  __shared__ int s_wtot[WAVES];
 
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform by construction; say so
@@ -138,12 +139,20 @@ void rows_kernel(RowsArgs p) {
 
   CATS_RSTAMP(0);
   const int row0 = (blockIdx.x * WAVES + wave) * R;
-  int row[R];
+  int row[R];   // weight row to read
+  int orow[R];  // position in the outputs
   bool on[R];
 #pragma unroll
   for (int r = 0; r < R; r++) {
-    row[r] = row0 + r < p.N ? row0 + r : p.N - 1;
+    orow[r] = row0 + r < p.N ? row0 + r : p.N - 1;
+    row[r] = orow[r];
     on[r] = row0 + r < p.N;
+    if (MODE == kUpIndex) {
+      const long long j = p.row_idx[orow[r]];
+      const bool ok = j >= 0 && j < (long long)p.w_rows;
+      row[r] = __builtin_amdgcn_readfirstlane(ok ? (int)j : 0);
+      on[r] = on[r] && __builtin_amdgcn_readfirstlane((int)ok) != 0;  // an entry outside the matrix reads nothing and yields 0
+    }
   }
 
   // Staging order matters: memory returns are counted in issue order, so the x loads go out first, then the
@@ -164,7 +173,7 @@ void rows_kernel(RowsArgs p) {
       if (i < B * nchv && b < p.nb && v < p.row_vecs) xpre[k] = p.x[(size_t)b * p.row_vecs + v];
     }
   }
-  if (MODE != kUp) rows_issue<R, CB, FULL>(p.w, row, on, 0, p, lane, wv);
+  if (MODE != kUp && MODE != kUpIndex) rows_issue<R, CB, FULL>(p.w, row, on, 0, p, lane, wv);
   if (XLDS) {
 #pragma unroll
     for (int k = 0; k < kXPre; k++) {
@@ -202,7 +211,19 @@ void rows_kernel(RowsArgs p) {
   bool act[R][B];      // per batch row flag
   bool any[R];         // union over the batch
 
-  if (MODE == kUp) {
+  if (MODE == kUpIndex) {
+    // every list entry is fetched; what multiplies the dot product comes from the compact scale vector (or is 1)
+    const st* sc = (const st*)p.scale;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+      any[r] = on[r];
+#pragma unroll
+      for (int b = 0; b < B; b++) {
+        act[r][b] = on[r] && b < p.nb;
+        a[r][b] = sc ? DT::tof(sc[orow[r]]) : 1.f;
+      }
+    }
+  } else if (MODE == kUp) {
     const st* ain = (const st*)p.a_in;
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -258,12 +279,7 @@ void rows_kernel(RowsArgs p) {
 #pragma unroll
           for (int b = 0; b < B; b++)
             if (b < p.nb) {
-              if (MODE == kGate && p.a_out) {
-                st* dst = (st*)p.a_out + (size_t)b * p.N + row[r];
-                // read back by another workgroup (the one that builds the list): device-coherent store
-                if (p.idx_out) __hip_atomic_store(dst, DT::fromf(a[r][b]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                else *dst = DT::fromf(a[r][b]);
-              }
+              if (MODE == kGate && p.a_out) ((st*)p.a_out)[(size_t)b * p.N + row[r]] = DT::fromf(a[r][b]);
               if (p.flag_out) p.flag_out[(size_t)b * p.N + row[r]] = act[r][b] ? 1 : 0;
             }
         }
@@ -277,20 +293,34 @@ void rows_kernel(RowsArgs p) {
   }
 
   CATS_RSTAMP(2);
-  if (MODE == kGateUp || MODE == kUp) {
+  if (MODE == kGateUp || MODE == kUp || MODE == kUpIndex) {
     float u[R][B];
     rows_dot<DT, B, R, CB, FULL, XLDS>(MODE == kGateUp ? p.w2 : p.w, row, any, xs, p.x, p, lane, wv, false, u);
     if (lane == 0) {
 #pragma unroll
       for (int r = 0; r < R; r++)
-        if (on[r]) {
+        if (row0 + r < p.N) {
 #pragma unroll
           for (int b = 0; b < B; b++)
             if (b < p.nb) {
-              const float z = act[r][b] ? DT::rnd(a[r][b] * DT::rnd(u[r][b])) : 0.f;
-              const size_t o = (size_t)b * p.N + row[r];
-              if (p.z32_out && (MODE == kUp || any[r])) p.z32_out[o] = z;
-              if (p.zt_out) ((st*)p.zt_out)[o] = DT::fromf(z);
+              const size_t o = (size_t)b * p.N + orow[r];
+              if (MODE == kUpIndex) {
+                // fp32 all the way, one rounding at the store: dot product, bias of the weight row, activation, scale
+                float v = 0.f;
+                if (act[r][b]) {
+                  v = u[r][b];
+                  if (p.bias) v += DT::tof(((const st*)p.bias)[row[r]]);
+                  if (p.activation == 1) v = fmaxf(v, 0.f);
+                  else if (p.activation == 2) { v = fmaxf(v, 0.f); v = v * v; }
+                  else if (p.activation == 3) v = v / (1.f + expf(-v));
+                  v *= a[r][b];
+                }
+                ((st*)p.zt_out)[o] = DT::fromf(v);
+              } else {
+                const float z = act[r][b] ? DT::rnd(a[r][b] * DT::rnd(u[r][b])) : 0.f;
+                if (p.z32_out && (MODE == kUp || any[r])) p.z32_out[o] = z;
+                if (p.zt_out) ((st*)p.zt_out)[o] = DT::fromf(z);
+              }
             }
         }
     }
@@ -303,85 +333,101 @@ void rows_kernel(RowsArgs p) {
       const int nbytes = (p.N + 7) >> 3;
       if (threadIdx.x < kRowsPerBlock / 8) {
         const int byte = blockIdx.x * (kRowsPerBlock / 8) + threadIdx.x;
-        if (byte < nbytes) {
-          const uint8_t m8 = (uint8_t)(s_maskbits >> (8 * threadIdx.x));
-          if (MODE == kGate && p.idx_out) __hip_atomic_store(&p.mask_out[byte], m8, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          else p.mask_out[byte] = m8;
-        }
+        if (byte < nbytes) p.mask_out[byte] = (uint8_t)(s_maskbits >> (8 * threadIdx.x));
       }
     }
   }
+}
 
-  if (MODE == kGate) {
-    if (p.idx_out == nullptr) return;
-    // Last workgroup to arrive turns the mask bytes into an ascending index list: one byte (8 neurons) per thread
-    // and pass, popcount + wave prefix sum + LDS prefix over the waves for the rank, bit expansion for the entries.
-    // No release / acquire fences (at agent scope they write back and invalidate the whole L2): the activations and
-    // mask bytes were stored device-coherently above, each wave waits for its own stores to be acknowledged, the
-    // barrier joins the waves, then the arrival counter is bumped; the last workgroup reads with coherent loads.
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      // Two levels: atomics on one address are served one after the other (about 12 ns each), which for a thousand
-      // workgroups would cost more than the gate pass.  Workgroups count into 64 counters on separate lines; the
-      // last one of each counts into the top one.
-      constexpr uint32_t kSub = 64;
-      const uint32_t sub = blockIdx.x % kSub;
-      const uint32_t members = (gridDim.x - sub + kSub - 1) / kSub;
-      uint32_t* sc = p.arrive_sub + sub * 32;
-      bool last = false;
-      if (__hip_atomic_fetch_add(sc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1u) {
-        __hip_atomic_store(sc, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const uint32_t used = gridDim.x < kSub ? gridDim.x : kSub;
-        last = __hip_atomic_fetch_add(p.arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == used - 1u;
-      }
-      s_last = last;
+// Mask bytes -> ascending index list, the matching activations, and the count.  Runs after the gate kernel on the same
+// stream (the launch boundary orders it after every mask byte and activation).  Each workgroup takes a contiguous
+// range of mask bytes; where its part of the list starts is the number of set bits before the range, which it counts
+// itself from the mask (a few KiB, served from cache) -- so there is no dependence between workgroups.  Inside the range:
+// one byte (8 neurons) per thread and pass, popcount, wave prefix sum, LDS prefix over the waves, bit expansion.
+struct CompactArgs {
+  const uint8_t* mask;   // ceil(N / 8) bytes
+  const void* a;         // (N,) activations in the storage type, 16-byte aligned, readable up to a multiple of 16 bytes
+  int64_t* idx_out;      // (>= count,)
+  void* vals_out;        // optional (>= count,) storage type
+  int32_t* count_out;
+  int N;
+  int bytes_per_group;   // mask bytes per workgroup
+};
+
+template <int ESZ>
+__global__ __launch_bounds__(256) void compact_kernel(CompactArgs p) {
+  typedef typename std::conditional<ESZ == 2, uint16_t, uint32_t>::type st;
+  constexpr int WAVES = 4;
+  __shared__ int s_wtot[WAVES];
+  __shared__ int s_base;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  const int nbytes = (p.N + 7) >> 3;
+  const int byte0 = blockIdx.x * p.bytes_per_group;
+  const int byte1 = min(nbytes, byte0 + p.bytes_per_group);
+  auto bits_of = [&](int byte) -> uint32_t {
+    uint32_t bits = p.mask[byte];
+    const int rem = p.N - byte * 8;
+    if (rem < 8) bits &= (1u << rem) - 1u;
+    return bits;
+  };
+  constexpr int kVecs = ESZ * 8 / 16;  // 16-byte vectors holding the 8 activations of one mask byte
+  const u32x4* avec = (const u32x4*)p.a;
+  const int nvec = (p.N * ESZ + 15) / 16;  // whole vectors that hold activations (the buffer is at least that long)
+  // A mask byte and its 8 activations are fetched together, and the first pass's fetch goes out before anything else:
+  // with the count of the bits before the range that makes one memory round trip for the usual one-pass range.
+  u32x4 av[kVecs];
+  uint32_t bits = 0u;
+  auto fetch = [&](int byte) {
+#pragma unroll
+    for (int q = 0; q < kVecs; q++) {
+      const int v = byte * kVecs + q;
+      av[q] = (p.vals_out && byte < byte1 && v < nvec) ? avec[v] : zero4();
     }
+    bits = byte < byte1 ? bits_of(byte) : 0u;
+  };
+  fetch(byte0 + tid);
+  // set bits before this workgroup's range (the last workgroup goes on to the end and so has the total)
+  const bool last_group = blockIdx.x == gridDim.x - 1;
+  int before = 0;
+  for (int byte = tid; byte < byte0; byte += 256) before += __popc(bits_of(byte));
+  before = (int)wave_sum((float)before);  // below 2^24: exact in fp32
+  if (lane == 0) s_wtot[wave] = before;
+  __syncthreads();
+  if (tid == 0) s_base = s_wtot[0] + s_wtot[1] + s_wtot[2] + s_wtot[3];
+  __syncthreads();
+  int base = s_base;
+  for (int b0 = byte0; b0 < byte1; b0 += 256) {
+    const int byte = b0 + tid;
+    if (b0 != byte0) fetch(byte);
+    const int pc = __popc(bits);
+    const int incl = wave_scan_inclusive(pc, lane);
+    __syncthreads();  // s_wtot of the previous pass (or of the count above) has been read
+    if (lane == kWave - 1) s_wtot[wave] = incl;
     __syncthreads();
-    if (!s_last) return;
-    const st* aall = (const st*)p.a_out;
-    const int nbytes = (p.N + 7) >> 3;
-    int base = 0;
-    for (int b0 = 0; b0 < nbytes; b0 += kThreads) {
-      const int byte = b0 + threadIdx.x;
-      uint32_t bits = 0;
-      if (byte < nbytes) bits = __hip_atomic_load(&p.mask_out[byte], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const int pc = __popc(bits);
-      const int incl = wave_scan_inclusive(pc, lane);
-      if (lane == kWave - 1) s_wtot[wave] = incl;
-      __syncthreads();
-      int before = 0, total = 0;
+    int pre = 0, total = 0;
 #pragma unroll
-      for (int w = 0; w < WAVES; w++) {
-        const int c = s_wtot[w];
-        if (w < wave) before += c;
-        total += c;
-      }
-      const int o = base + before + incl - pc;
-      // the 8 neurons of the byte, unrolled: all activation loads go out before the first store
-      st v8[8];
+    for (int w = 0; w < WAVES; w++) {
+      const int c = s_wtot[w];
+      if (w < wave) pre += c;
+      total += c;
+    }
+    const int o = base + pre + incl - pc;
 #pragma unroll
-      for (int k = 0; k < 8; k++) {
-        v8[k] = DT::fromf(0.f);
-        if (p.vals_out && ((bits >> k) & 1u))
-          v8[k] = __hip_atomic_load(&aall[byte * 8 + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-#pragma unroll
-      for (int k = 0; k < 8; k++) {
-        if ((bits >> k) & 1u) {
-          const int r = o + __popc(bits & ((1u << k) - 1u));
-          p.idx_out[r] = byte * 8 + k;
-          if (p.vals_out) ((st*)p.vals_out)[r] = v8[k];
+    for (int k = 0; k < 8; k++) {
+      if ((bits >> k) & 1u) {
+        const int r = o + __popc(bits & ((1u << k) - 1u));
+        p.idx_out[r] = byte * 8 + k;
+        if (p.vals_out) {
+          const uint32_t word = av[k * ESZ / 16][(k * ESZ % 16) / 4];
+          ((st*)p.vals_out)[r] = ESZ == 2 ? (st)(word >> (16 * (k & 1))) : (st)word;
         }
       }
-      base += total;
-      __syncthreads();
     }
-    if (threadIdx.x == 0) {
-      *p.count_out = base;
-      __hip_atomic_store(p.arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    base += total;
   }
+  if (last_group && tid == 0) *p.count_out = base;
 }
 
 }  // namespace cats

@@ -296,6 +296,59 @@ at::Tensor cats_down_flag_op(const at::Tensor& x, const at::Tensor& weight, cons
   return out;
 }
 
+// gather_gemv / gather_gemv_elemul_indirect_index_2d: x (B, H), weight (Z, H), idx (M,) int64 -> (B, M)
+at::Tensor cats_up_index_op(const at::Tensor& x, const at::Tensor& weight, const at::Tensor& idx, const c10::optional<at::Tensor>& bias,
+                            const c10::optional<at::Tensor>& scale, int64_t activation) {
+  check_dev(x, "x");
+  TORCH_CHECK(x.dim() == 2, "flash_gemv.cats_up_index: x must be (batch, N)");
+  const int64_t B = x.size(0), H = x.size(1), Z = weight.size(0), M = idx.numel();
+  TORCH_CHECK(B >= 1 && B <= 8, "flash_gemv.cats_up_index: batch of ", B, " rows is not supported (1..8)");
+  check_weight(weight, x, Z, H, "weight");
+  check_dev(idx, "idx");
+  TORCH_CHECK(idx.scalar_type() == at::kLong && idx.dim() == 1, "flash_gemv.cats_up_index: idx must be a 1-D int64 tensor");
+  const void* bp = nullptr;
+  const void* sp = nullptr;
+  if (bias.has_value() && bias->defined()) {
+    check_dev(*bias, "bias");
+    TORCH_CHECK(bias->scalar_type() == x.scalar_type() && bias->numel() == Z, "flash_gemv.cats_up_index: bias must be (Z,) of x's dtype");
+    bp = bias->data_ptr();
+  }
+  if (scale.has_value() && scale->defined()) {
+    check_dev(*scale, "scale");
+    TORCH_CHECK(scale->scalar_type() == x.scalar_type() && scale->numel() == M, "flash_gemv.cats_up_index: scale must have one entry per index, in x's dtype");
+    sp = scale->data_ptr();
+  }
+  at::Tensor out = at::empty({B, M}, x.options());
+  check_status(cats_up_index(x.data_ptr(), weight.data_ptr(), idx.data_ptr<int64_t>(), (int)M, bp, sp, (int)activation, out.data_ptr(), (int)B,
+                             (int)H, (int)Z, dtype_code(x), current_stream(x)),
+               "cats_up_index");
+  return out;
+}
+
+// gather_transposed_gemv / gather_transposed_gemv_indirect_index_2d: z (B, M), weight (Z, N) neuron-major, idx (M,) -> (B, N)
+at::Tensor cats_down_index_op(const at::Tensor& z, const at::Tensor& weight, const at::Tensor& idx, const c10::optional<at::Tensor>& bias) {
+  check_dev(z, "x");
+  TORCH_CHECK(z.dim() == 2, "flash_gemv.cats_down_index: x must be (batch, M)");
+  const int64_t B = z.size(0), M = z.size(1), Z = weight.size(0), H = weight.size(1);
+  TORCH_CHECK(B >= 1 && B <= 8, "flash_gemv.cats_down_index: batch of ", B, " rows is not supported (1..8)");
+  check_weight(weight, z, Z, H, "weight (neuron-major)");
+  check_dev(idx, "idx");
+  TORCH_CHECK(idx.scalar_type() == at::kLong && idx.dim() == 1 && idx.numel() == M, "flash_gemv.cats_down_index: idx must be int64 with one entry per column of x");
+  const void* bp = nullptr;
+  if (bias.has_value() && bias->defined()) {
+    check_dev(*bias, "bias");
+    TORCH_CHECK(bias->scalar_type() == z.scalar_type() && bias->numel() == H, "flash_gemv.cats_down_index: bias must be (N,) of x's dtype");
+    bp = bias->data_ptr();
+  }
+  at::Tensor out = at::empty({B, H}, z.options());
+  hipStream_t s = current_stream(z);
+  Workspace& ws = workspace(z, (int)B, (int)H, (int)Z, s);
+  check_status(cats_down_index(z.data_ptr(), weight.data_ptr(), idx.data_ptr<int64_t>(), (int)M, bp, out.data_ptr(), (int)B, (int)H, (int)Z,
+                               dtype_code(z), ws.buf.data_ptr(), ws.bytes, s),
+               "cats_down_index");
+  return out;
+}
+
 // Whole CATS MLP in two launches: x (B,1,H) or (B,H); wgate, wup, wdown_t all (I,H).  Returns x-shaped y.
 at::Tensor cats_mlp_op(const at::Tensor& x, const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown_t, const double threshold) {
   check_dev(x, "x");
@@ -392,6 +445,8 @@ TORCH_LIBRARY(flash_gemv, m) {
   // HIP replacements for the Triton wrappers and the fused two-launch MLP
   m.def("cats_up_flag", cats_up_flag_op);
   m.def("cats_down_flag", cats_down_flag_op);
+  m.def("cats_up_index", cats_up_index_op);
+  m.def("cats_down_index", cats_down_index_op);
   m.def("cats_mlp", cats_mlp_op);
   m.def("cats_mlp_norm_residual", cats_mlp_norm_residual_op);
   m.def("cats_up_down", cats_up_down_op);

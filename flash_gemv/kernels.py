@@ -6,8 +6,9 @@ through ``torch.ops.flash_gemv`` -- nothing here imports Triton.
 Flag-based pair (the path the reference publishes numbers for):
   gather_gemv_elemul_flag_3d      kernels.py:208-254   sparse up,   z = x_1 * (x . wup[j]) where flagged
   gather_transposed_gemv_flag_3d  kernels.py:416-462   sparse down, y = sum_j z[j] * weight[j, :]
-Index-list (DejaVu-style) family (kernels.py:639-695, 1022-1094, 1236-1334): the sorted index list is
-scattered into a flag row and the same two kernels run; results are gathered back to the list order.
+Index-list (DejaVu-style) family (kernels.py:639-695, 1022-1094, 1236-1334): the kernels read the index list and
+fetch exactly the listed weight rows (cats_up_index / cats_down_index); inputs and outputs stay compact, aligned
+with the list.
 """
 from typing import Optional
 
@@ -47,16 +48,16 @@ def gather_transposed_gemv_flag_3d(x: torch.Tensor, weight: torch.Tensor, idx: t
     return torch.ops.flash_gemv.cats_down_flag(x, weight, idx.contiguous())
 
 
-def _flags_from_index(idx: torch.Tensor, rows: int, width: int) -> torch.Tensor:
-    flags = torch.zeros(rows, width, dtype=torch.bool, device=idx.device)
-    flags[:, idx] = True
-    return flags
+_ACTIVATIONS = {"id": 0, "relu": 1, "squared_relu": 2, "swish": 3}
 
 
 def gather_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Tensor, bias: Optional[torch.Tensor] = None,
                 activation: str = "id") -> torch.Tensor:
-    """y = activation(x @ weight[idx, :].T + bias[idx]); x (batch, N), weight (Z, N), idx (M,) -> (batch, M)."""
-    assert activation in ["id", "relu", "squared_relu", "swish"]
+    """y = activation(x @ weight[idx, :].T + bias[idx]); x (batch, N), weight (Z, N), idx (M,) -> (batch, M).
+
+    The kernel reads the list and fetches exactly those rows (reference kernels.py:484-695): fp32 accumulation, bias,
+    activation, one rounding at the store."""
+    assert activation in _ACTIVATIONS
     Z, N = weight.shape
     batch, _ = x.shape
     assert x.shape == (batch, N)
@@ -65,49 +66,46 @@ def gather_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Tensor, bias: 
     if weight.stride(1) > 1:
         weight = weight.contiguous()
     assert x.dtype == weight.dtype, f"Input and weight must have the same dtype, got {x.dtype} and {weight.dtype}"
-    flags = _flags_from_index(idx, batch, Z)
-    ones = torch.ones(batch, Z, dtype=x.dtype, device=x.device)
-    y = torch.ops.flash_gemv.cats_up_flag(x, ones, weight, flags)[:, idx]
     if bias is not None:
+        bias = bias.contiguous()
         assert bias.shape == (Z,), "Incompatible dimensions in between weight and bias"
-        y = y + bias[idx]
-    if activation == "relu":
-        y = torch.relu(y)
-    elif activation == "squared_relu":
-        y = torch.relu(y) ** 2
-    elif activation == "swish":
-        y = torch.nn.functional.silu(y)
-    return y
+        assert x.dtype == bias.dtype, f"Input and bias must have the same dtype, got {x.dtype} and {bias.dtype}"
+    return torch.ops.flash_gemv.cats_up_index(x, weight, idx.contiguous(), bias, None, _ACTIVATIONS[activation])
 
 
 def gather_transposed_gemv(x: torch.Tensor, weight: torch.Tensor, idx: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """y = x @ weight[idx, :] + bias; x (batch, M), weight (Z, N), idx (M,) -> (batch, N)."""
+    """y = x @ weight[idx, :] + bias; x (batch, M), weight (Z, N), idx (M,) -> (batch, N) in x.dtype (kernels.py:1022-1094).
+    Duplicate entries of idx add up, as they do with the reference's atomic adds."""
     Z, N = weight.shape
-    batch, M = x.shape
-    assert idx.shape == (M,)
+    (M,) = idx.shape
+    batch, _ = x.shape
+    assert x.shape == (batch, M)
+    x = x.contiguous()
     if weight.stride(1) > 1:
         weight = weight.contiguous()
     assert x.dtype == weight.dtype, f"Input and weight must have the same dtype, got {x.dtype} and {weight.dtype}"
-    flags = _flags_from_index(idx, batch, Z)
-    dense = torch.zeros(batch, Z, dtype=x.dtype, device=x.device)
-    dense[:, idx] = x
-    y = torch.ops.flash_gemv.cats_down_flag(dense, weight, flags)
     if bias is not None:
-        y = y + bias
-    return y
+        bias = bias.contiguous()
+        assert bias.shape == (N,), "Incompatible dimensions in between weight and bias"
+        assert x.dtype == bias.dtype, f"Input and bias must have the same dtype, got {x.dtype} and {bias.dtype}"
+    return torch.ops.flash_gemv.cats_down_index(x, weight, idx.contiguous(), bias)
 
 
 def gather_gemv_elemul_indirect_index_2d(x: torch.Tensor, x_1: torch.Tensor, Wup: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
-    """y = x_1 * (x @ Wup[idx, :].T); x (1, N), x_1 (M,) compact activations, idx (M,) -> (1, M)."""
+    """y = x_1 * (x @ Wup[idx, :].T); x (1, N), x_1 (M,) compact activations, idx (M,) -> (1, M) (kernels.py:1236-1274):
+    the multiply happens in fp32 inside the kernel, before the one rounding."""
     _, N = Wup.shape
     beam_width, _ = x.shape
+    (M,) = idx.shape
     assert x.shape[1] == N
     assert beam_width == 1
-    return gather_gemv(x, Wup, idx) * x_1
+    if Wup.stride(1) > 1:
+        Wup = Wup.contiguous()
+    return torch.ops.flash_gemv.cats_up_index(x.contiguous(), Wup, idx.contiguous(), None, x_1.contiguous().view(-1), 0)
 
 
 def gather_transposed_gemv_indirect_index_2d(x: torch.Tensor, weight: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
-    """y = x @ weight[idx, :]; x (beam, M), idx (M,) -> (beam, N) in x.dtype."""
+    """y = x @ weight[idx, :]; x (beam, M), idx (M,) -> (beam, N) in x.dtype (kernels.py:1276-1325)."""
     (M,) = idx.shape
     assert x.shape[1] == M
     return gather_transposed_gemv(x.contiguous(), weight, idx)

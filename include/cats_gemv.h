@@ -80,7 +80,8 @@ int cats_gate_flag(const void* x, const void* wgate, void* a_out, uint8_t* flag_
 
 /* Same gate pass, B == 1, that also emits the compact active set: idx_out[0..count) ascending neuron
  * indices (int64), vals_out[0..count) the matching activations in dtype, *count_out (device int32) the
- * count.  The list is built by the last workgroup to finish, with wave ballots and a prefix sum.
+ * count.  Two launches: the gate pass (activations and mask bytes into the workspace), then a small kernel that
+ * turns the mask bytes into the list with popcounts, wave prefix sums and bit expansion.
  * Replaces fuse_gemv_cmp (flash_gemv.py:3-4; fuse_gemv_cmp_cuda.cu:43-88,1962-1977), whose list is in
  * atomic arrival order and whose count lives in a process-global managed int. */
 int cats_gate_compact(const void* x, const void* wgate, void* vals_out, int64_t* idx_out, int32_t* count_out,
@@ -106,6 +107,23 @@ int cats_up_flag(const void* x, const void* wup, const void* a, const uint8_t* f
  * Exactly one of y_f32 / y_out must be non-NULL.  Needs a workspace. */
 int cats_down_flag(const void* z, const void* wdown_t, const uint8_t* flag, float* y_f32, void* y_out,
                    int B, int H, int I, int dtype, void* ws, size_t ws_bytes, void* stream);
+
+/* Index-list ("DejaVu") up projection: out[b, m] = scale[m] * act(x[b,:] . w[idx[m],:] + bias[idx[m]]) for the M entries
+ * of idx (int64 weight-row numbers, any order, duplicates allowed; an entry outside [0, Z) yields 0).  Only the listed
+ * rows of w (Z, H) are read.  bias (Z,) and scale (M,) are optional, in dtype; activation 0 = identity, 1 = relu,
+ * 2 = squared relu, 3 = swish; fp32 throughout with one rounding at the store.  out (B, M) in dtype.
+ * Replaces gather_gemv (flash_gemv/flash_gemv/kernels.py:484-695) and, with scale = the compact gate activations,
+ * gather_gemv_elemul_indirect_index_2d (kernels.py:1112-1150, 1236-1274). */
+int cats_up_index(const void* x, const void* w, const int64_t* idx, int M, const void* bias, const void* scale, int activation,
+                  void* out, int B, int H, int Z, int dtype, void* stream);
+
+/* Index-list down projection: y[b,:] = sum over m of z[b, m] * wdown_t[idx[m], :] (+ bias), z (B, M) aligned with the list,
+ * wdown_t (Z, H) neuron-major, bias (H,) optional.  Duplicate entries add up (as the reference's atomics do), entries
+ * outside [0, Z) contribute nothing.  y_out (B, H) in dtype, fp32 accumulation in a fixed order.  Needs a workspace.
+ * Replaces gather_transposed_gemv (kernels.py:753-1094) and gather_transposed_gemv_indirect_index_2d
+ * (kernels.py:1204-1234, 1276-1325). */
+int cats_down_index(const void* z, const void* wdown_t, const int64_t* idx, int M, const void* bias, void* y_out,
+                    int B, int H, int Z, int dtype, void* ws, size_t ws_bytes, void* stream);
 
 /* Gate + sparse up in one pass: out[b,j] = active ? round(a * up) : 0 in dtype, flag_out optional.
  * Replaces fuse_gemv_flag_gemv (flash_gemv.py:9-10; fuse_gemv_cmp_cuda.cu:715-784,2006-2022). */

@@ -108,6 +108,41 @@ def torch_layer_tail(h, norm_weight, eps, wgate, wup, wdown, threshold):
     return h + y
 
 
+def torch_gather_gemv(x, weight, idx, bias=None, activation="id", scale=None):
+    """Index-list up projection, the reference's formula y = activation(x @ weight[idx, :].T + bias[idx])
+    (flash_gemv/flash_gemv/kernels.py:645-652, activations :46-66 of the kernel's epilogue: relu, squared relu, swish),
+    optionally times the compact gate activations (gather_gemv_elemul_indirect_index_2d, kernels.py:1242-1250).
+    Evaluated in fp32 with one rounding to x.dtype at the end, as the Triton kernels accumulate and store."""
+    xf, wf = _cpu(x).float(), _cpu(weight).float()
+    idx = _cpu(idx).long()
+    y = xf @ wf[idx, :].t()
+    if bias is not None:
+        y = y + _cpu(bias).float()[idx]
+    if activation == "relu":
+        y = torch.relu(y)
+    elif activation == "squared_relu":
+        y = torch.relu(y) ** 2
+    elif activation == "swish":
+        y = y * torch.sigmoid(y)
+    elif activation != "id":
+        raise ValueError(activation)
+    if scale is not None:
+        y = y * _cpu(scale).float().view(1, -1)
+    return y.to(x.dtype)
+
+
+def torch_gather_transposed_gemv(x, weight, idx, bias=None):
+    """Index-list down projection, the reference's formula y = weight[idx, :]^T @ x + bias (kernels.py:1028-1034): every
+    entry of idx contributes x[:, m] * weight[idx[m], :], so duplicate entries add up (the reference adds with atomics,
+    kernels.py:842-850).  fp32 with one rounding to x.dtype at the end (kernels.py:1061-1094)."""
+    xf, wf = _cpu(x).float(), _cpu(weight).float()
+    idx = _cpu(idx).long()
+    y = xf @ wf[idx, :]
+    if bias is not None:
+        y = y + _cpu(bias).float().view(1, -1)
+    return y.to(x.dtype)
+
+
 def torch_flags(x_1, threshold):
     """flash_gemv/flash_gemv/__init__.py:41,46 -- computed in x_1's dtype, the scalar is cast to it."""
     return torch.abs(x_1) > threshold

@@ -253,7 +253,9 @@ def test_up_down_given_the_gate_activations(oracle, H, I, B, dtype):
 
 
 def test_gate_compact_list(oracle):
-    for (H, I, dtype) in ((64, 96, torch.float16), (512, 1000, torch.bfloat16), (4096, 2048, torch.float16), (256, 300, torch.float32)):
+    # 11008 neurons = 1376 mask bytes = six workgroups of the list kernel; 2051 ends inside a byte; 20000 is three passes per workgroup
+    for (H, I, dtype) in ((64, 96, torch.float16), (512, 1000, torch.bfloat16), (4096, 2048, torch.float16), (256, 300, torch.float32),
+                          (4096, 11008, torch.float16), (128, 2051, torch.bfloat16), (64, 20000, torch.float16), (64, 150000, torch.float16)):
         m = make_mlp(H, I, 1, dtype, seed=31)
         d = dev(m)
         ws = _ws(1, H, I)
@@ -261,13 +263,174 @@ def test_gate_compact_list(oracle):
             a_ref, _ = capi.gate_flag(d["x"], d["wg"], -1.0)
             mags = a_ref.float().abs().flatten()
             t = -1.0 if q == 0.0 else (float("inf") if q > 1 else float(torch.quantile(mags, q)))
-            for _ in range(2):  # twice: the arrival counter must reset itself
+            for _ in range(2):  # twice: nothing may be left behind in the workspace
                 vals, idx, n = capi.gate_compact(d["x"], d["wg"], t, ws)
                 a, flag = capi.gate_flag(d["x"], d["wg"], t)
                 want_idx, want_n = oracle.c_compact(flag[0])
                 assert n == want_n == int(flag.sum())
                 assert torch.equal(idx[:n].cpu(), want_idx), "index list is not ascending nonzero(mask)"
                 assert torch.equal(vals[:n].cpu(), a[0].cpu()[want_idx])
+
+
+INDEX_LIST = [
+    # H (row length), Z (rows of the weight), M (list length), B, dtype
+    (4096, 11008, 5500, 1, torch.float16), (4096, 2048, 700, 2, torch.bfloat16), (520, 1000, 333, 3, torch.float16),
+    (260, 333, 333, 4, torch.float32), (4096, 512, 1, 1, torch.float16), (2048, 640, 77, 8, torch.bfloat16), (64, 96, 200, 2, torch.float32),
+]
+
+
+@pytest.mark.parametrize("H,Z,M,B,dtype", INDEX_LIST)
+def test_index_list_up_and_down(oracle, H, Z, M, B, dtype):
+    """cats_up_index / cats_down_index through the C ABI against the reference's formulas (oracle.torch_gather_gemv /
+    torch_gather_transposed_gemv): sorted lists, unsorted lists with duplicates (M may exceed Z), bias, every activation,
+    the compact scale vector, entries outside the matrix, the empty list."""
+    g = torch.Generator().manual_seed(H + Z + M)
+    x = torch.randn(B, H, generator=g).to(dtype)
+    w = (torch.randn(Z, H, generator=g) * 0.05).to(dtype)
+    wd = (torch.randn(Z, H, generator=g) * 0.05).to(dtype)
+    bias_up = torch.randn(Z, generator=g).to(dtype)
+    bias_dn = torch.randn(H, generator=g).to(dtype)
+    sorted_idx = torch.sort(torch.randperm(Z, generator=g)[: min(M, Z)]).values
+    any_idx = torch.randint(0, Z, (M,), generator=g)
+    ws = _ws(B, H, Z)
+    dx, dw, dwd = x.cuda(), w.cuda(), wd.cuda()
+    for idx in (sorted_idx, any_idx):
+        di = idx.cuda()
+        scale = torch.randn(idx.numel(), generator=g).to(dtype)
+        for act in ("id", "relu", "squared_relu", "swish"):
+            for b_, sc in ((None, None), (bias_up, None), (None, scale), (bias_up, scale)):
+                got = capi.up_index(dx, dw, di, None if b_ is None else b_.cuda(), None if sc is None else sc.cuda(), act)
+                want = oracle.torch_gather_gemv(x, w, idx, b_, act, sc)
+                close(got.cpu(), want, dtype)
+        z = (torch.randn(B, idx.numel(), generator=g) * 0.5).to(dtype)
+        for b_ in (None, bias_dn):
+            got = capi.down_index(z.cuda(), dwd, di, ws, None if b_ is None else b_.cuda())
+            want = oracle.torch_gather_transposed_gemv(z, wd, idx, b_)
+            close(got.cpu(), want, dtype)
+            again = capi.down_index(z.cuda(), dwd, di, ws, None if b_ is None else b_.cuda())
+            assert torch.equal(got, again), "index-list down is not repeatable bit for bit"
+    # entries outside [0, Z) give 0 (up) / contribute nothing (down) instead of reading outside the matrix
+    bad = any_idx.clone()
+    bad[::3] = Z + 5
+    bad[1::7] = -1
+    ok = (bad >= 0) & (bad < Z)
+    got = capi.up_index(dx, dw, bad.cuda())
+    want = oracle.torch_gather_gemv(x, w, bad.clamp(0, Z - 1))
+    want[:, ~ok] = 0
+    close(got.cpu(), want, dtype)
+    z = (torch.randn(B, M, generator=g) * 0.5).to(dtype)
+    got = capi.down_index(z.cuda(), dwd, bad.cuda(), ws)
+    close(got.cpu(), oracle.torch_gather_transposed_gemv(z[:, ok], wd, bad[ok]), dtype)
+    # the empty list: y = bias, or zeros
+    empty = torch.zeros(0, dtype=torch.int64, device="cuda")
+    ze = torch.zeros(B, 0, dtype=dtype, device="cuda")
+    assert torch.equal(capi.down_index(ze, dwd, empty, ws).cpu(), torch.zeros(B, H, dtype=dtype))
+    assert torch.equal(capi.down_index(ze, dwd, empty, ws, bias_dn.cuda()).cpu(), bias_dn.expand(B, H))
+    assert capi.up_index(dx, dw, empty).shape == (B, 0)
+
+
+def test_index_list_package_functions(oracle):
+    """The reference's Python names on top of the index-list kernels: gather_gemv (batch 1..4, bias, activations),
+    gather_transposed_gemv, the *_indirect_index_2d pair and both composites, against the oracle's formulas."""
+    import flash_gemv as fg
+    from flash_gemv import kernels as K
+
+    g = torch.Generator().manual_seed(12)
+    H, Z = 1024, 1536
+    dtype = torch.float16
+    w = (torch.randn(Z, H, generator=g) * 0.05).to(dtype)
+    wdt = (torch.randn(Z, H, generator=g) * 0.05).to(dtype)
+    bias = torch.randn(Z, generator=g).to(dtype)
+    for batch in (1, 2, 3, 4):
+        x = torch.randn(batch, H, generator=g).to(dtype)
+        idx = torch.sort(torch.randperm(Z, generator=g)[:500]).values
+        for act in ("id", "relu", "squared_relu", "swish"):
+            for b_ in (None, bias):
+                got = K.gather_gemv(x.cuda(), w.cuda(), idx.cuda(), None if b_ is None else b_.cuda(), act)
+                close(got.cpu(), oracle.torch_gather_gemv(x, w, idx, b_, act), dtype)
+        z = (torch.randn(batch, 500, generator=g) * 0.5).to(dtype)
+        hb = torch.randn(H, generator=g).to(dtype)
+        close(K.gather_transposed_gemv(z.cuda(), wdt.cuda(), idx.cuda()).cpu(), oracle.torch_gather_transposed_gemv(z, wdt, idx), dtype)
+        close(K.gather_transposed_gemv(z.cuda(), wdt.cuda(), idx.cuda(), hb.cuda()).cpu(), oracle.torch_gather_transposed_gemv(z, wdt, idx, hb), dtype)
+    x = torch.randn(1, H, generator=g).to(dtype)
+    x1 = torch.randn(500, generator=g).to(dtype)
+    close(K.gather_gemv_elemul_indirect_index_2d(x.cuda(), x1.cuda(), w.cuda(), idx.cuda()).cpu(), oracle.torch_gather_gemv(x, w, idx, scale=x1), dtype)
+    z1 = (oracle.torch_gather_gemv(x, w, idx).float() * x1.float()).to(dtype)
+    want = oracle.torch_gather_transposed_gemv(z1, wdt, idx)
+    close(K.mistral_mlp_partial_sparse(x.cuda(), x1.cuda(), w.cuda(), wdt.cuda(), idx.cuda()).cpu(), want, dtype)
+    close(K.mistral_mlp_sparse_direct_index_2d(x.cuda(), x1.cuda(), w.cuda(), wdt.cuda(), idx.cuda()).cpu(), want, dtype)
+    # the whole-MLP composites: gate in torch, sorted active list, index-list up and down == the flag-based path
+    wg_t = (torch.randn(H, Z, generator=g) * 0.02).to(dtype)
+    t = 0.05
+    a = fg.flag_gemv_gemv_dejavu(x.cuda(), wg_t.cuda(), w.cuda(), wdt.cuda(), t)
+    b = fg.flag_gemv_gemv_fuse_dejavu(x.cuda(), wg_t.cuda(), w.cuda(), wdt.cuda(), t)
+    c = fg.flag_gemv_gemv_triton(x.cuda().view(1, 1, H), wg_t.cuda(), w.cuda(), wdt.cuda(), t)
+    close(a.cpu(), c.view(1, H).cpu(), dtype)
+    close(b.cpu(), c.view(1, H).cpu(), dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_mask_boundaries_on_the_device(oracle, dtype):
+    """Crafted activations around the threshold, on every copy of the rule the kernels carry.
+
+    With x = e_0 the gate pre-activation of neuron j is exactly wgate[j, 0], so the stored activation a_j =
+    round(silu(wgate[j, 0])) can be steered: the first column holds a ladder of values whose activations straddle
+    candidate thresholds.  Thresholds are then taken FROM the stored activations of the kernel -- a == t exactly, the
+    neighbouring representable values on either side, -t, 0, a value below every |a| and +inf -- and the flags of
+    (i) the gate kernel (wave-per-row at 1 and 2 rows, matrix-core at 4 and 8 rows), (ii) the single-pass MLP kernel,
+    (iii) the two-kernel MLP path and (iv) cats_up_down, which derives flags from a supplied a, must all equal
+    torch.abs(a) > t and the C oracle's comparison, bit for bit (experiments/models/sparse_silu/ugly_utils.py:897,
+    flash_gemv/flash_gemv/__init__.py:41,46)."""
+    H, I = 4096, 512
+    g = torch.Generator().manual_seed(9)
+    ladder = torch.cat([torch.linspace(-6, 6, I - 8), torch.tensor([0.0, -0.0, 1e-7, -1e-7, 6e-8, 1.0, -1.0, 0.5])])
+    wg = torch.zeros(I, H)
+    wg[:, 0] = ladder
+    wg = wg.to(dtype)
+    wu = (torch.randn(I, H, generator=g) * 0.02).to(dtype)
+    wdt = (torch.randn(I, H, generator=g) * 0.02).to(dtype)
+    for B in (1, 2, 4, 8):
+        x = torch.zeros(B, H)
+        x[:, 0] = 1.0
+        x = x.to(dtype)
+        dx, dwg, dwu, dwdt = x.cuda(), wg.cuda(), wu.cuda(), wdt.cuda()
+        ws = _ws(B, H, I)
+        a0, _ = capi.gate_flag(dx, dwg, -1.0)
+        a0 = a0.cpu()
+        torch.testing.assert_close(a0[0].float(), torch.nn.functional.silu(wg[:, 0].float()), **A_TOL[dtype])  # a = round(silu(w)) for x = e_0
+        mags = torch.unique(a0[0].float().abs())
+        mid = mags[mags.numel() // 2]          # a positive value that some neuron's |a| equals exactly
+        itype = torch.int32 if dtype == torch.float32 else torch.int16
+        mid_bits = mid.to(dtype).view(itype)
+        up1 = (mid_bits + 1).view(dtype).float()   # neighbouring representable values of the storage type
+        dn1 = (mid_bits - 1).view(dtype).float()
+        small = mags[mags > 0].min()
+        cands = [float(mid), float(up1), float(dn1), -float(mid), 0.0, -0.0, float(small), float(small) / 2, -1.0, float(mags.max()), float("inf"),
+                 float(mid) * (1 + 1e-4), float(mid) * (1 - 1e-4)]   # the last two are not representable in 16 bits: the threshold itself gets rounded
+        for t in cands:
+            a, flag = capi.gate_flag(dx, dwg, t)
+            want = torch.abs(a) > t                      # torch's own comparison on the kernel's activations, on the device
+            assert torch.equal(flag, want), f"gate flags differ from |a| > t at t={t} B={B}"
+            tr = oracle.c_round(dtype, t)
+            assert torch.equal(flag.cpu(), a.cpu().float().abs() > tr), f"gate flags differ from the C oracle's rule at t={t}"
+            _, f_mlp, cnt = capi.mlp(dx, dwg, dwu, dwdt, t, ws, want_flag=True, want_count=True)
+            assert torch.equal(f_mlp, want) and int(cnt) == int(want.any(dim=0).sum()), f"MLP flags differ at t={t} B={B}"
+            try:
+                capi.set_tuning(0, 0, 0, 1)
+                _, f_two, cnt2 = capi.mlp(dx, dwg, dwu, dwdt, t, ws, want_flag=True, want_count=True)
+                y_two = capi.up_down(dx, a, dwu, dwdt, t, ws)
+            finally:
+                capi.set_tuning(0, 0, 0, 0)
+            assert torch.equal(f_two, want) and int(cnt2) == int(want.any(dim=0).sum()), f"two-kernel MLP flags differ at t={t} B={B}"
+            # cats_up_down derives its flags from the supplied a: same output as feeding it a with the dropped entries zeroed
+            # and a threshold below everything that is left
+            y_a = capi.up_down(dx, a, dwu, dwdt, t, ws)
+            a_masked = torch.where(want, a, torch.zeros_like(a))
+            flag_masked = a_masked != 0
+            z = capi.up_flag(dx, dwu, a_masked, flag_masked)
+            y_ref = capi.down_flag(z, dwdt, flag_masked, ws)
+            close(y_a.cpu(), y_ref.cpu(), dtype)
+            close(y_two.cpu(), y_ref.cpu(), dtype)
 
 
 def test_sparse_up_and_down_ops(oracle):

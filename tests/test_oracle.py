@@ -328,3 +328,58 @@ def test_oracle_reproduces_the_frozen_vectors_bit_for_bit(oracle):
         y_t, _, dead = oracle.torch_cats_mlp(c["x"].float(), c["wg"].float(), c["wu"].float(), c["wd"].float(), c["t"])
         if torch.equal(~dead, c["flag"]):
             torch.testing.assert_close(y_t, c["y"].float(), rtol=1e-2, atol=2e-3 * max(1.0, float(c["y"].float().abs().max())))
+
+
+def test_index_list_projections_brute_force_and_special_cases(oracle):
+    """The index-list pair is pinned by plain float64 loops on a small case, by reducing to the dense library GEMV when
+    the list is every row once, by linearity for duplicate entries, and by a wrong formula shown to fail."""
+    g = torch.Generator().manual_seed(3)
+    B, N, Z = 2, 24, 17
+    x = torch.randn(B, N, generator=g)
+    w = torch.randn(Z, N, generator=g)
+    bias_up = torch.randn(Z, generator=g)
+    idx = torch.tensor([5, 0, 16, 5, 9])     # unsorted, one duplicate
+    scale = torch.randn(idx.numel(), generator=g)
+    for act in ("id", "relu", "squared_relu", "swish"):
+        got = oracle.torch_gather_gemv(x, w, idx, bias_up, act, scale)
+        want = torch.zeros(B, idx.numel(), dtype=torch.float64)
+        for b in range(B):
+            for m, j in enumerate(idx.tolist()):
+                v = sum(float(x[b, k]) * float(w[j, k]) for k in range(N)) + float(bias_up[j])
+                if act == "relu":
+                    v = max(v, 0.0)
+                elif act == "squared_relu":
+                    v = max(v, 0.0) ** 2
+                elif act == "swish":
+                    v = v / (1.0 + math.exp(-v))
+                want[b, m] = v * float(scale[m])
+        torch.testing.assert_close(got.double(), want, rtol=1e-5, atol=1e-5)
+    # bias indexed by position instead of by weight row (a plausible slip) is a different function
+    wrong = x @ w[idx].t() + bias_up[: idx.numel()]
+    assert not torch.allclose(oracle.torch_gather_gemv(x, w, idx, bias_up), wrong, atol=1e-3)
+    # the whole matrix once: the library's dense GEMV
+    every = torch.arange(Z)
+    torch.testing.assert_close(oracle.torch_gather_gemv(x, w, every), torch.nn.functional.linear(x, w))
+
+    H = 11
+    wd = torch.randn(Z, H, generator=g)
+    z = torch.randn(B, idx.numel(), generator=g)
+    bias_dn = torch.randn(H, generator=g)
+    got = oracle.torch_gather_transposed_gemv(z, wd, idx, bias_dn)
+    want = torch.zeros(B, H, dtype=torch.float64)
+    for b in range(B):
+        for h in range(H):
+            want[b, h] = sum(float(z[b, m]) * float(wd[j, h]) for m, j in enumerate(idx.tolist())) + float(bias_dn[h])
+    torch.testing.assert_close(got.double(), want, rtol=1e-5, atol=1e-5)
+    # duplicates add: listing row 5 twice with z1, z2 equals listing it once with z1 + z2
+    merged_idx = torch.tensor([5, 0, 16, 9])
+    merged_z = torch.stack([z[:, 0] + z[:, 3], z[:, 1], z[:, 2], z[:, 4]], dim=1)
+    torch.testing.assert_close(got, oracle.torch_gather_transposed_gemv(merged_z, wd, merged_idx, bias_dn), rtol=1e-5, atol=1e-5)
+    # the whole matrix once: z @ wd, and the sorted active list reproduces the flag-based sparse down of the C oracle
+    zz = torch.randn(B, Z, generator=g)
+    torch.testing.assert_close(oracle.torch_gather_transposed_gemv(zz, wd, every), zz @ wd, rtol=1e-5, atol=1e-5)
+    flag = torch.zeros(B, Z, dtype=torch.bool)
+    flag[:, merged_idx] = True
+    live = torch.nonzero(flag[0]).flatten()
+    dense = oracle.c_sparse_down(torch.where(flag, zz, torch.zeros_like(zz)), wd, flag)
+    torch.testing.assert_close(oracle.torch_gather_transposed_gemv(zz[:, live], wd, live), dense, rtol=1e-5, atol=1e-5)
