@@ -310,3 +310,83 @@ def test_two_streams_with_their_own_workspaces_do_not_interfere():
     for i in range(6):
         assert torch.equal(got1[i], want1[i]), f"stream 1, call {i}"
         assert torch.equal(got8[i], want8[i]), f"stream 2, call {i}"
+
+
+def test_bounded_soak_of_every_hot_entry_point_stays_bitwise_stable():
+    """A few hundred calls cycling batch sizes 1 / 2 / 4 / 8, the whole-MLP entry points, the compact-list gate and the
+    index-list pair, two alternating inputs through the same workspaces, two streams with their own workspaces, and a
+    HIP graph replayed between eager calls.  Every result is compared bit for bit with the first result of its kind and
+    the run stops at the first mismatch: nothing a call leaves behind (partial sums, mask bytes, counters, LDS-sized
+    scratch) may leak into a later call, whatever ran in between."""
+    import flash_gemv as fg
+    from flash_gemv import kernels as K
+
+    H, I = 4096, 1536
+    g = torch.Generator(device="cuda").manual_seed(33)
+    rn = lambda *s: torch.randn(*s, generator=g, device="cuda")
+    wg, wu, wdt = (rn(I, H) * 0.02).half(), (rn(I, H) * 0.02).half(), (rn(I, H) * 0.02).half()
+    nw = (1 + 0.1 * rn(H)).half()
+    t = 0.04
+    inputs = {B: [rn(B, 1, H).half(), (rn(B, 1, H) * 1.5).half()] for B in (1, 2, 4, 8)}
+    idx_out = torch.zeros(I, dtype=torch.int64, device="cuda")
+    vals = torch.zeros(1, 1, I, dtype=torch.float16, device="cuda")
+
+    def run(kind, B, which):
+        x = inputs[B][which]
+        if kind == "mlp":
+            return fg.cats_mlp(x, wg, wu, wdt, t)
+        if kind == "tail":
+            return fg.cats_mlp_norm_residual(x, nw, 1e-5, wg, wu, wdt, t)
+        if kind == "updown":
+            a = torch.empty(B, 1, I, dtype=torch.float16, device="cuda")
+            f = torch.empty(B, 1, I, dtype=torch.bool, device="cuda")
+            fg.fuse_gemv_flag_local(x, wg, a, f, t)
+            return fg.gemv_gemv_triton(x, a, wu, wdt, t)
+        if kind == "compact":  # batch 1 only
+            n = fg.fuse_gemv_cmp(inputs[1][which], wg, vals, idx_out, t)
+            return torch.cat([idx_out[:n].float(), vals.flatten()[:n].float()])
+        if kind == "index":    # index-list up and down over the list the compact gate produced
+            n = fg.fuse_gemv_cmp(inputs[1][which], wg, vals, idx_out, t)
+            x2 = inputs[B][which].view(B, H)
+            z = K.gather_gemv(x2, wu, idx_out[:n].clone(), None, "swish")
+            return K.gather_transposed_gemv(z, wdt, idx_out[:n].clone())
+        raise ValueError(kind)
+
+    kinds = ["mlp", "tail", "updown", "compact", "index"]
+    first = {}
+    # a graph holding one single-pass call and one batch-8 call, replayed between the eager calls on another stream
+    gx1, gx8 = inputs[1][0].clone(), inputs[8][1].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        fg.cats_mlp(gx1, wg, wu, wdt, t)
+        fg.cats_mlp(gx8, wg, wu, wdt, t)
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            gy1 = fg.cats_mlp(gx1, wg, wu, wdt, t)
+            gy8 = fg.cats_mlp(gx8, wg, wu, wdt, t)
+    torch.cuda.synchronize()
+    want_g1 = fg.cats_mlp(gx1, wg, wu, wdt, t).clone()
+    want_g8 = fg.cats_mlp(gx8, wg, wu, wdt, t).clone()
+    other = torch.cuda.Stream()
+    calls = 0
+    for it in range(60):
+        for B in (1, 2, 4, 8):
+            kind = kinds[(it + B) % len(kinds)]
+            if kind == "compact" and B != 1:
+                kind = "mlp"
+            which = (it // 2 + B) % 2
+            stream = other if it % 3 == 1 else torch.cuda.current_stream()
+            with torch.cuda.stream(stream):
+                got = run(kind, B, which)
+            stream.synchronize()
+            key = (kind, B, which, it % 3 == 1)   # per stream: each stream has its own workspace, results must not depend on it
+            base = first.setdefault((kind, B, which), got.clone())
+            assert torch.equal(got, base), f"iteration {it}: {key} differs from the first result of its kind"
+            calls += 1
+        if it % 4 == 0:
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(gy1, want_g1) and torch.equal(gy8, want_g8), f"iteration {it}: graph replay differs from the eager result"
+    assert calls == 240
