@@ -1,12 +1,16 @@
 """Build the gfx950 kernels and the torch op library in-tree.
 
-Two shared objects come out of this:
+Three shared objects come out of this:
 
 * ``cats_amd/lib/libcats_gemv.so`` -- the HIP kernels behind the C ABI of ``include/cats_gemv.h``.
   No torch in it: plain pointers, sizes and a stream.
 * ``flash_gemv/_C.so`` -- a thin ``TORCH_LIBRARY(flash_gemv, m)`` shim that unpacks tensors, picks the
   current HIP stream, owns a cached workspace and calls the C ABI.  It takes the place of the reference's
   ``flash_gemv/_C*.so`` (built there by ``flash_gemv/setup.py:51-97`` with nvcc).
+
+* ``cats_amd/lib/libcats_gemv_timing.so`` -- the kernel library compiled with ``-DCATS_TIMING``: every workgroup
+  stamps the wall clock at its phase boundaries into a caller-supplied buffer.  Only ``cats_amd.phase_stamps``
+  loads it.
 
 Run ``python -m cats_amd.build`` (hipcc cross-compiles for gfx950 without a GPU).
 """
@@ -23,6 +27,7 @@ CSRC = ROOT / "cats_amd" / "csrc"
 OBJ = ROOT / "build" / "obj"
 LIB_DIR = ROOT / "cats_amd" / "lib"
 KERNEL_LIB = LIB_DIR / "libcats_gemv.so"
+TIMING_LIB = LIB_DIR / "libcats_gemv_timing.so"   # same kernels with per-workgroup wall-clock stamps (-DCATS_TIMING)
 TORCH_LIB = ROOT / "flash_gemv" / "_C.so"
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -45,20 +50,24 @@ def _run(cmd: list[str]) -> None:
         print(err, file=sys.stderr)
 
 
-def build_kernels(jobs: int = 4) -> Path:
-    OBJ.mkdir(parents=True, exist_ok=True)
+def build_kernels(jobs: int = 4, timing: bool = False) -> Path:
+    """The kernel library; with ``timing`` the instrumented twin that ``cats_amd.phase_stamps`` loads (never the product)."""
+    obj = OBJ / "timing" if timing else OBJ
+    out = TIMING_LIB if timing else KERNEL_LIB
+    extra = ["-DCATS_TIMING"] if timing else []
+    obj.mkdir(parents=True, exist_ok=True)
     LIB_DIR.mkdir(parents=True, exist_ok=True)
     units = [
-        (CSRC / "cats_inst.hip", OBJ / "cats_inst_f16.o", ["-DCATS_DT=F16"]),
-        (CSRC / "cats_inst.hip", OBJ / "cats_inst_bf16.o", ["-DCATS_DT=BF16"]),
-        (CSRC / "cats_inst.hip", OBJ / "cats_inst_f32.o", ["-DCATS_DT=F32"]),
-        (CSRC / "cats_api.hip", OBJ / "cats_api.o", []),
+        (CSRC / "cats_inst.hip", obj / "cats_inst_f16.o", ["-DCATS_DT=F16"]),
+        (CSRC / "cats_inst.hip", obj / "cats_inst_bf16.o", ["-DCATS_DT=BF16"]),
+        (CSRC / "cats_inst.hip", obj / "cats_inst_f32.o", ["-DCATS_DT=F32"]),
+        (CSRC / "cats_api.hip", obj / "cats_api.o", []),
     ]
-    cmds = [[HIPCC, *HIP_FLAGS, *defs, "-c", str(src), "-o", str(obj)] for src, obj, defs in units]
+    cmds = [[HIPCC, *HIP_FLAGS, *extra, *defs, "-c", str(src), "-o", str(o)] for src, o, defs in units]
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(_run, cmds))
-    _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(KERNEL_LIB), *[str(u[1]) for u in units]])
-    return KERNEL_LIB
+    _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(out), *[str(u[1]) for u in units]])
+    return out
 
 
 def build_torch_shim() -> Path:
@@ -86,6 +95,7 @@ def build_torch_shim() -> Path:
 def build_all() -> None:
     print(f"[cats_amd.build] kernels  -> {build_kernels()}")
     print(f"[cats_amd.build] torch op -> {build_torch_shim()}")
+    print(f"[cats_amd.build] stamped  -> {build_kernels(timing=True)}")
 
 
 if __name__ == "__main__":

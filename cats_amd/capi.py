@@ -30,6 +30,14 @@ class CatsError(RuntimeError):
     pass
 
 
+def use_library(path) -> None:
+    """Bind another build of the kernel library (the stamped one, say).  Only before the first call into it."""
+    global _LIB_PATH
+    if _lib is not None:
+        raise RuntimeError("the kernel library is already loaded")
+    _LIB_PATH = Path(path)
+
+
 def lib() -> ctypes.CDLL:
     global _lib
     if _lib is None:

@@ -38,7 +38,7 @@ long long* g_tbuf_fused = nullptr;
 
 constexpr int kMaxSlabs = 128;
 constexpr int kKernelBatch = 8;  // rows one launch handles; the entry points take up to CATS_MAX_BATCH rows in passes of this many
-constexpr size_t kCounterBytes = 1024 + 64 * 128;  // uint32 words: done[0..127] | arrive 128 | count 192 | 64 arrival sub-counters, one per 128-byte line
+constexpr size_t kCounterBytes = 1024 + 64 * 128;  // reserved head of the workspace; no kernel keeps state in it any more
 
 __global__ void fill_zero_kernel(u32x4* p, size_t n16) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) p[i] = zero4();
@@ -53,8 +53,7 @@ struct WsLayout {
 constexpr int kMaxGroups = 64;  // neuron groups of the sparse down kernel; bounds the partial-sum scratch
 
 // The carving depends on (H, I) only -- every region is sized for kKernelBatch rows -- so calls with
-// different batch sizes can share one workspace and the region that must stay zero (the counters) never
-// moves onto bytes another call has dirtied.
+// different batch sizes can share one workspace.  Nothing in it has to survive from one call to the next.
 WsLayout ws_layout(int H, int I) {
   WsLayout l;
   const int B = kKernelBatch;

@@ -61,14 +61,14 @@ typedef enum {
 int cats_version(void);
 const char* cats_status_string(int status);
 
-/* Workspace: scratch for the mask words, the fp32 intermediate z, the fp32 output accumulator and a few
- * counters.  Replaces the per-call cudaMalloc/cudaFree pairs of the reference
+/* Workspace: scratch for the per-workgroup partial sums, the mask bytes, the fp32 intermediate z and the
+ * gate activations of the list-building call.  Replaces the per-call cudaMalloc/cudaFree pairs of the reference
  * (fuse_gemv_cmp_cuda.cu:2351-2354,2402-2403).  The caller allocates cats_workspace_bytes() once (256-byte
  * aligned), runs cats_workspace_init() once (it zero-fills with a kernel), and then passes the same buffer to
- * every call; each call leaves the parts that must start at zero zeroed again.  The size and the carving
- * depend on (H, I) only (B is checked, every region holds CATS_MAX_BATCH rows), so one workspace serves every
- * batch size of one layer shape; for another (H, I) use another workspace or initialise again.  One workspace
- * serves one stream at a time. */
+ * every call; no call relies on what an earlier call left in it.  The size and the carving depend on (H, I)
+ * only (B is checked; every region holds the 8 rows of one pass over the weights, and a call with 9..16 rows
+ * reuses them pass by pass), so one workspace serves every batch size of one layer shape; for another (H, I)
+ * use another workspace or initialise again.  One workspace serves one stream at a time. */
 size_t cats_workspace_bytes(int B, int H, int I);
 int cats_workspace_init(void* ws, size_t ws_bytes, void* stream);
 
