@@ -15,9 +15,10 @@
 // bitwise reproducible run to run.  The two kernels are ordered by the stream, which is the only cross-workgroup
 // synchronisation there is.
 //
-// Inside the workgroup the producer / consumer hand-off runs through LDS: a row wave writes z, then the slot state;
-// the LDS unit executes one wave's accesses in issue order, so a down wave that reads "live" and then z reads the z
-// that was written before it.  Down waves poll with s_sleep; all waves of a workgroup are resident together, so the
+// Inside the workgroup the producer / consumer hand-off runs through LDS: a row wave writes z, a release fence, then
+// the slot state (relaxed workgroup-scope atomic); a down wave reads the state (relaxed atomic), an acquire fence,
+// then z.  Both fences name the LDS address space only, so they cost an s_waitcnt lgkmcnt(0) and never wait for the
+// weight loads in flight.  Down waves poll with s_sleep; all waves of a workgroup are resident together, so the
 // producers always make progress.
 #pragma once
 #include "cats_device.h"
@@ -108,8 +109,8 @@ struct DownBatch {
 
 // Where the down waves read what the row waves publish: slot i is neuron row0 + i.
 struct FusedSlots {
-  volatile int* state;    // [n] FusedSlot
-  volatile float* z;      // [n][B]
+  int* state;    // [n] FusedSlot; written and read with workgroup-scope atomics
+  float* z;      // [n][B]; ordered against state by LDS-only release / acquire fences
   int row0, n;
 };
 
@@ -130,10 +131,8 @@ __device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const Fu
   while (head < sl.n) {
     const int idx = head + lane;
     const bool in = idx < sl.n;  // never read past the slot array
-    const int st_ = in ? sl.state[idx] : kSlotPending;  // past the end counts as pending: it ends the decided prefix
-    int zv[B];
-#pragma unroll
-    for (int b = 0; b < B; b++) zv[b] = in ? __builtin_bit_cast(int, sl.z[idx * B + b]) : 0;
+    // past the end counts as pending: it ends the decided prefix
+    const int st_ = in ? __hip_atomic_load(&sl.state[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : kSlotPending;
     const uint64_t pend = __ballot(st_ == kSlotPending);
     uint64_t live = __ballot(st_ == kSlotLive);
     const int ready = pend ? __builtin_ctzll(pend) : kWave;  // slots head .. head + ready - 1 are decided
@@ -142,6 +141,11 @@ __device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const Fu
       __builtin_amdgcn_s_sleep(1);
       continue;
     }
+    // acquire side of the hand-off (LDS only): the z of every slot seen decided above is read after its state
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    int zv[B];
+#pragma unroll
+    for (int b = 0; b < B; b++) zv[b] = in ? __builtin_bit_cast(int, sl.z[idx * B + b]) : 0;
     if (ready < kWave) live &= (1ull << ready) - 1ull;
 #pragma unroll
     for (int u = 0; u < RB; u++) {
@@ -208,8 +212,8 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
 
   u32x4* xs = s_fused;                                       // [B][nchv]
   FusedSlots sl;
-  sl.state = (volatile int*)(s_fused + B * nchv);          // [rpw]
-  sl.z = (volatile float*)(sl.state + ((p.rpw + 3) & ~3));  // [rpw][B]
+  sl.state = (int*)(s_fused + B * nchv);          // [rpw]
+  sl.z = (float*)(sl.state + ((p.rpw + 3) & ~3));  // [rpw][B]
   sl.row0 = row0;
   sl.n = n;
 
@@ -344,8 +348,9 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
         const int slot = row - row0;
 #pragma unroll
         for (int b = 0; b < B; b++) sl.z[slot * B + b] = z[b];
-        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): z is in LDS before the state says so
-        sl.state[slot] = any ? kSlotLive : kSlotDead;
+        // release side (LDS only, so the gate rows in flight are not waited for): z is in LDS before the state says so
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __hip_atomic_store(&sl.state[slot], any ? kSlotLive : kSlotDead, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
       cur = nxt;
       nxt = neuron_of(__builtin_amdgcn_readfirstlane(pend));
