@@ -44,6 +44,26 @@ __global__ void fill_zero_kernel(u32x4* p, size_t n16) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) p[i] = zero4();
 }
 
+// Number of neurons flagged in any of the B rows of flags (B, I): the count of a call that ran as several passes.
+__global__ __launch_bounds__(1024) void union_count_kernel(const uint8_t* __restrict__ flags, int B, int I, int32_t* count_out) {
+  __shared__ int s_part[16];
+  int k = 0;
+  for (int j = threadIdx.x; j < I; j += blockDim.x) {
+    uint32_t on = 0;
+    for (int b = 0; b < B; b++) on |= flags[(size_t)b * I + j];
+    k += on != 0;
+  }
+  k = (int)wave_sum((float)k);  // at most I / 16 per wave, far below 2^24: exact in fp32
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x >> 6;
+  if (lane == 0) s_part[wave] = k;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int tot = 0;
+    for (int w = 0; w < (int)(blockDim.x >> 6); w++) tot += s_part[w];
+    *count_out = tot;
+  }
+}
+
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct WsLayout {
@@ -657,12 +677,23 @@ int cats_gate_up(const void* x, const void* wgate, const void* wup, void* out, u
 int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, float* y_f32,
              uint8_t* flag_out, int32_t* count_out, int B, int H, int I, int dtype, float threshold, void* ws,
              size_t ws_bytes, void* stream) {
-  if (count_out && B > kKernelBatch) return CATS_ERR_BATCH;  // the count is that of one pass
   const size_t sz = esz(dtype);
-  return in_passes(B, [&](size_t b0, int nb) {
+  const bool union_count = count_out && B > kKernelBatch;  // a pass counts its own rows only: count the union of the flags instead
+  if (union_count && !flag_out) {
+    // no flags asked for: the passes write them into the workspace region of the row-major intermediate, which no MLP pass uses
+    WsLayout l;
+    if (int st = check_common(kKernelBatch, H, I, dtype)) return st;
+    if (int st = check_ws(ws, ws_bytes, H, I, l)) return st;
+    flag_out = (uint8_t*)ws + l.zt;  // 8 * I * 4 bytes hold CATS_MAX_BATCH * I flags
+  }
+  int st = in_passes(B, [&](size_t b0, int nb) {
     return mlp_pass(at_cbytes(x, b0 * H * sz), wgate, wup, wdown_t, at_bytes(y_out, b0 * H * sz), (float*)at_bytes((void*)y_f32, b0 * H * 4),
-                    (uint8_t*)at_bytes((void*)flag_out, b0 * I), count_out, nb, H, I, dtype, threshold, ws, ws_bytes, stream);
+                    (uint8_t*)at_bytes((void*)flag_out, b0 * I), union_count ? nullptr : count_out, nb, H, I, dtype, threshold, ws, ws_bytes,
+                    stream);
   });
+  if (st || !union_count) return st;
+  union_count_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(flag_out, B, I, count_out);
+  return hipGetLastError() == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
 }
 
 int cats_mlp_stage(int stage, const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,

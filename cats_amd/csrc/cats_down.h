@@ -239,6 +239,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   // semantics): one fp32 atomic per column per workgroup.
   constexpr int FB = B < 4 ? B : 4;  // batch rows folded per pass
   __syncthreads();  // the list and z are dead from here on; their LDS is reused
+  CATS_STAMP(4);
 #pragma unroll
   for (int b0 = 0; b0 < B; b0 += FB) {
     if (b0 > 0) __syncthreads();  // the previous pass has been read
@@ -280,6 +281,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
     }
   }
 
+  CATS_STAMP(5);
   if (p.count_out && blockIdx.x == 0) {  // not on the hot path: total popcount of the mask
     __syncthreads();  // s_red is reused below; the fold above may still be reading it
     int k = 0;

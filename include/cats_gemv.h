@@ -134,8 +134,9 @@ int cats_gate_up(const void* x, const void* wgate, const void* wup, void* out, u
  * takes its neurons through gate, up and down and leaves (B,H) partial sums, then a reduction over the workgroups;
  * more rows (and y_f32 mode): gate+up kernel, then sparse down kernel.
  *   y_out != NULL : (B,H) in dtype;  y_f32 != NULL : fp32 accumulate into the caller's pre-zeroed (B,H).
- * flag_out (B,I) optional.  count_out (device int32, optional, B <= 8 only) receives the number of neurons fetched
- * (union over the batch).
+ * flag_out (B,I) optional.  count_out (device int32, optional) receives the number of neurons active in any row of the
+ * batch (for up to 8 rows that is the number of neurons fetched; 9..16 rows fetch per pass and one small kernel counts
+ * the union of the flags afterwards).
  * Replaces flag_gemv_gemv_atomic, fuse_gemv_gemv_gemv, fuse_gemv_flag_gemv_gemv (flash_gemv.py:12-16,30-31;
  * fuse_gemv_cmp_cuda.cu:786-1244,2196-2253) and the composite gemv_gemv_triton / flag_gemv_gemv_triton
  * (flash_gemv/flash_gemv/__init__.py:38-48). */

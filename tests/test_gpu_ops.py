@@ -127,8 +127,8 @@ def test_bad_arguments_raise_not_exit():
     w = torch.zeros(96, 64, dtype=torch.float16, device="cuda")
     with pytest.raises(RuntimeError, match="batch"):
         fg.cats_mlp(x, w, w, w, 0.1)
-    with pytest.raises(RuntimeError, match="batch"):   # the active count is per pass of 8 rows
-        fg.cats_mlp_stats(x[:9], w, w, w, 0.1)
+    _, flags9, count9 = fg.cats_mlp_stats(x[:9], w, w, w, 0.1)   # two passes: the count is the union of the flags
+    assert int(count9) == int(flags9.view(9, -1).any(dim=0).sum())
     with pytest.raises(RuntimeError, match="must be"):
         fg.cats_mlp(x[:1], w, w[:, :32].contiguous(), w, 0.1)
     with pytest.raises(RuntimeError, match="dtype"):

@@ -48,7 +48,7 @@ def check_mlp_case(oracle, m, t, *, tag, ws=None, expect_flip_free=False):
     ws = ws or _ws(B, H, I)
 
     a, flag = capi.gate_flag(d["x"], d["wg"], t)
-    y, flag2, count = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=B <= 8)
+    y, flag2, count = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
     if (I * m["x"].element_size()) % 16 == 0:
         y_rm = capi.mlp_rowmajor_down(d["x"], d["wg"], d["wu"], d["wd"], t, ws)
     else:  # rows of the (H, I) down weight are not 16-byte aligned: rejected, not mis-read
@@ -63,7 +63,7 @@ def check_mlp_case(oracle, m, t, *, tag, ws=None, expect_flip_free=False):
     assert torch.equal(flag, want_flag), f"{tag}: flag != (|a| > t) on the kernel's own a"
     assert torch.equal(flag2, flag), f"{tag}: the fused MLP pass and the gate pass disagree on flags"
     union = flag.any(dim=0)
-    if count is not None:  # batches above 8 rows run as two passes and report no count
+    if count is not None:  # above 8 rows (two passes) this is the union of the flags, counted by one more small kernel
         assert int(count.item()) == int(union.sum()), f"{tag}: active count {int(count.item())} != {int(union.sum())}"
     # the C oracle's rule on the same activations (independent of torch's scalar casting)
     tr = oracle.c_round(dtype, t)
@@ -733,8 +733,29 @@ def test_batch_above_sixteen_is_an_error_not_a_crash():
     z = lambda *s: torch.zeros(*s, dtype=torch.float16, device="cuda")
     with pytest.raises(capi.CatsError, match="batch"):
         capi.mlp(z(17, 512), z(64, 512), z(64, 512), z(64, 512), 0.1, _ws(8, 512, 64))
-    with pytest.raises(capi.CatsError, match="batch"):   # the count is per pass: not offered above 8 rows
-        capi.mlp(z(9, 512), z(64, 512), z(64, 512), z(64, 512), 0.1, _ws(8, 512, 64), want_count=True)
+
+
+def test_active_count_above_eight_rows_is_the_union_over_both_passes(oracle):
+    """9..16 rows run as two passes of 8; the count must still be the number of neurons active in any row, whether or
+    not the caller asks for the flags (without them the passes write the flags into the workspace)."""
+    for B, H, I in ((9, 512, 200), (16, 1024, 333), (12, 4096, 11008)):
+        m = make_mlp(H, I, B, torch.float16, seed=B)
+        d = dev(m)
+        t = float(torch.quantile(torch.nn.functional.silu(m["x"].float() @ m["wg"].float().t()).abs().flatten()[::7], 0.95))
+        ws = _ws(B, H, I)
+        y, flag, count = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
+        cnt_only = torch.full((1,), -1, dtype=torch.int32, device="cuda")
+        y2 = torch.empty_like(y)
+        L = capi.lib()
+        st = L.cats_mlp(capi._p(d["x"]), capi._p(d["wg"]), capi._p(d["wu"]), capi._p(d["wdt"]), capi._p(y2), None, None, capi._p(cnt_only),
+                        B, H, I, capi.F16, t, capi._p(ws.buf), ws.nbytes, capi._stream(d["x"]))
+        assert st == 0
+        torch.cuda.synchronize()
+        want = int(flag.cpu().bool().any(dim=0).sum())
+        assert 0 < want < I
+        assert int(count.item()) == want
+        assert int(cnt_only.item()) == want
+        assert torch.equal(y, y2)
 
 
 def test_reference_recipe_shapes(oracle):
