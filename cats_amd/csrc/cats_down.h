@@ -96,7 +96,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   extern __shared__ __attribute__((aligned(16))) float s_dyn[];  // 8- and 16-byte LDS accesses below: a 4-byte-aligned base makes every one of them a slow unaligned access
   // dynamic LDS, streaming phase: [chunk] int list | [B][chunk] z in storage type (indexed by j - j0)
   //                               | 16-bit types: [chunk / 2][B] packed z pairs in list order
-  // afterwards reused for the fold: [nwaves / 2][B][VEC][64] float
+  // afterwards reused for the fold: [nwaves][min(B, 4)][64][VEC] float
   int* s_list = (int*)s_dyn;
   st* s_z = (st*)(s_dyn + p.chunk);
   uint32_t* s_zp = (uint32_t*)(s_dyn + p.chunk) + (B * p.chunk * sizeof(st) + 3) / 4;
@@ -230,44 +230,48 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   CATS_STAMP(2);
   // ---- 3. fold the waves through LDS -----------------------------------------------------------------------
   // Up to four batch rows at a time (16 waves x 4 x 2 KiB = 128 KiB of LDS): every wave writes its sums, one barrier,
-  // one thread per column adds the waves in wave order.  Eight batch rows take two such passes.  LDS layout of a pass:
-  // float (wave w, row b, pair q, lane l, k) at ((w * FB + b) * VEC/2 + q) * 128 + l * 2 + k  is column
-  // (slab * 64 + l) * VEC + 2 q + k  -- lanes write float2, consecutive lanes consecutive banks.
+  // one thread per four columns adds the waves in wave order.  Eight batch rows take two such passes.  LDS layout of a
+  // pass: the VEC sums of (wave w, row b, lane l) are the VEC / 4 float4 slots at ((w * FB + b) * 64 + l) * VEC / 4; for
+  // 16-bit types (two slots per lane) the two halves swap places in lanes 8..15 of every 16, which makes both the
+  // 16-byte writes (lane stride 32 bytes) and the reads (consecutive threads, consecutive slots) free of bank conflicts.
   // y_out mode: the folded sums go to the scratch partial [group][b][H]; the reduction launch that follows adds the
   // groups in order (a fixed summation order: bitwise reproducible output, nothing to zero between calls, no
   // cross-workgroup synchronisation inside this kernel).  y32 mode (the caller's fp32 accumulator, "atomic_gemv"
   // semantics): one fp32 atomic per column per workgroup.
   constexpr int FB = B < 4 ? B : 4;  // batch rows folded per pass
+  constexpr int kSlots = VEC / 4;    // float4 slots per lane and batch row
   __syncthreads();  // the list and z are dead from here on; their LDS is reused
   CATS_STAMP(4);
+  float4* s_red4 = (float4*)s_red;
 #pragma unroll
   for (int b0 = 0; b0 < B; b0 += FB) {
     if (b0 > 0) __syncthreads();  // the previous pass has been read
     {
-      float* dst = s_red + (size_t)wave * FB * kSlabCols + lane * 2;
+      const int swz = kSlots == 2 ? (lane >> 3) & 1 : 0;
 #pragma unroll
       for (int b = 0; b < FB; b++)
 #pragma unroll
-        for (int e = 0; e < VEC; e += 2) {
-          float2 v2 = {acc[b0 + b][e], acc[b0 + b][e + 1]};
-          *(float2*)(dst + b * kSlabCols + (e >> 1) * (2 * kWave)) = v2;
+        for (int h = 0; h < kSlots; h++) {
+          float4 v4 = {acc[b0 + b][4 * h], acc[b0 + b][4 * h + 1], acc[b0 + b][4 * h + 2], acc[b0 + b][4 * h + 3]};
+          s_red4[((size_t)(wave * FB + b) * kWave + lane) * kSlots + (h ^ swz)] = v4;
         }
     }
     __syncthreads();
     const int rows = min(FB, p.nb - b0);  // live batch rows of this pass (may be <= 0)
-    // One item = four consecutive columns of one batch row: two float2 per wave from LDS, one 16-byte store.  Whole
-    // sectors are written (a store of part of a 32-byte sector makes the memory side read the sector first).
+    // One item = one slot = four consecutive columns of one batch row: one float4 per wave from LDS, one 16-byte store.
+    // Consecutive threads take consecutive slots, so whole 32-byte sectors are written by neighbouring lanes (a store
+    // of part of a sector makes the memory side read the sector first).
     constexpr int kQuads = kSlabCols / 4;
     for (int it = tid; it < rows * kQuads; it += blockDim.x) {
       const int b = it / kQuads, r = it - b * kQuads;
-      const int l = r / (VEC / 4), h = r - l * (VEC / 4);  // lane that owned the columns, which quarter of its VEC
-      const float* src = s_red + b * kSlabCols + (2 * h) * (2 * kWave) + l * 2;
+      const int l = r / kSlots, ps = r - l * kSlots;                 // lane that owned the columns, physical slot
+      const int h = kSlots == 2 ? ps ^ ((l >> 3) & 1) : ps;          // which quarter of its VEC the slot holds
+      const float4* src = s_red4 + (size_t)b * kQuads + r;
       float4 s4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
+#pragma unroll 8
       for (int w = 0; w < nwaves; w++) {
-        const float2 lo = *(const float2*)(src + (size_t)w * FB * kSlabCols);
-        const float2 hi = *(const float2*)(src + (size_t)w * FB * kSlabCols + 2 * kWave);
-        s4.x += lo.x; s4.y += lo.y; s4.z += hi.x; s4.w += hi.y;
+        const float4 v4 = src[(size_t)w * FB * kQuads];
+        s4.x += v4.x; s4.y += v4.y; s4.z += v4.z; s4.w += v4.w;
       }
       const int col = (slab * kWave + l) * VEC + 4 * h;
       if (col < p.H) {  // H is a multiple of VEC, so a quad is inside or outside as a whole
