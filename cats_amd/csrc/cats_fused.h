@@ -250,7 +250,8 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       xs[i] = val;
     }
     for (int i = tid; i < p.rpw; i += kFusedThreads) sl.state[i] = kSlotPending;
-    if (tid == 0) s_ticket = 2 * RW;  // the first two neurons of every row wave are fixed, the rest go by ticket
+    // gate mode: the first two neurons of every row wave are fixed, the rest go by ticket; given activations: all by ticket
+    if (tid == 0) s_ticket = gate ? 2 * RW : 0;
     __syncthreads();
     if (p.norm_w) {
       // RMS norm of each batch row, in place in LDS: one wave adds a row's squares (fixed order), everyone rescales.
@@ -270,18 +271,113 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
     CATS_FSTAMP(tid == 0, 1);
   };
 
+  if (is_row_wave && !gate) {
+    // ---- row waves, gate activations given: the down waves have put them into the z slots while x was staged, so a
+    // wave knows whether a neuron is live from one LDS read.  It walks its tickets, publishes dead neurons at once and
+    // keeps the up rows of two live neurons (in blocks of CB chunks) in flight: the block of the next unit goes out
+    // before the current one is multiplied, both buffers always take a full block of loads (x, cached, when there is
+    // nothing left) so the wait for the older one is a fixed count.
+    stage([] {});
+    const int nblk = nchp / CB;
+    int irow = -1, iblk = 0;  // the neuron whose blocks are being issued
+    float ia[B];
+    bool iact[B];
+    auto next_live = [&]() -> int {
+      for (;;) {
+        int q = 0;
+        if (lane == 0) q = __hip_atomic_fetch_add(&s_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        q = __builtin_amdgcn_readfirstlane(q);
+        if (q >= n) return -1;
+        bool any = false;
+#pragma unroll
+        for (int b = 0; b < B; b++) {
+          ia[b] = sl.z[q * B + b];
+          iact[b] = b < p.nb && fabsf(ia[b]) > p.t;
+          any = any || iact[b];
+        }
+        any = __builtin_amdgcn_readfirstlane((int)any) != 0;
+        if (lane == 0 && p.flag_out) {
+#pragma unroll
+          for (int b = 0; b < B; b++)
+            if (b < p.nb) p.flag_out[(size_t)b * p.I + row0 + q] = iact[b] ? 1 : 0;
+        }
+        if (any) return row0 + q;
+        if (lane == 0) {
+#pragma unroll
+          for (int b = 0; b < B; b++) sl.z[q * B + b] = 0.f;
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+          __hip_atomic_store(&sl.state[q], kSlotDead, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+      }
+    };
+    // one unit = one block of one live neuron's up row; row < 0 = nothing left (the loads still go out, to x)
+    auto issue_next = [&](u32x4 (&buf)[CB], int& urow, int& ublk, float (&ua)[B], bool (&uact)[B]) {
+      if (irow < 0 || iblk == nblk) {
+        irow = next_live();
+        iblk = 0;
+      }
+      urow = irow;
+      ublk = irow >= 0 ? iblk++ : 0;
+#pragma unroll
+      for (int b = 0; b < B; b++) {
+        ua[b] = ia[b];
+        uact[b] = iact[b];
+      }
+      const u32x4* src = urow >= 0 ? p.wu + (size_t)urow * p.row_vecs : p.x;
+      fused_issue<CB, FULL>(src, ublk * CB, vlast, lane, buf);
+    };
+    float u[B];
+    auto consume = [&](const u32x4 (&buf)[CB], int urow, int ublk, const float (&ua)[B], const bool (&uact)[B]) {
+      if (urow < 0) return;  // wave-uniform
+      if (ublk == 0) {
+#pragma unroll
+        for (int b = 0; b < B; b++) u[b] = 0.f;
+      }
+      fused_dot<DT, B, CB>(buf, xs, nchv, ublk * CB, lane, u);
+      if (ublk != nblk - 1) return;
+      float z[B];
+#pragma unroll
+      for (int b = 0; b < B; b++) {
+        const float ub = wave_sum(u[b]);
+        z[b] = uact[b] ? DT::rnd(ua[b] * DT::rnd(ub)) : 0.f;
+      }
+      if (lane == 0) {
+        const int slot = urow - row0;
+#pragma unroll
+        for (int b = 0; b < B; b++) sl.z[slot * B + b] = z[b];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __hip_atomic_store(&sl.state[slot], kSlotLive, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+    };
+    u32x4 bufa[CB], bufb[CB];
+    int ra, ka, rb, kb;
+    float aa[B], ab[B];
+    bool ca[B], cb[B];
+    issue_next(bufa, ra, ka, aa, ca);
+    for (;;) {
+      issue_next(bufb, rb, kb, ab, cb);
+      consume(bufa, ra, ka, aa, ca);
+      if (rb < 0) break;
+      issue_next(bufa, ra, ka, aa, ca);
+      consume(bufb, rb, kb, ab, cb);
+      if (ra < 0) break;
+    }
+#ifdef CATS_TIMING
+    if (p.tbuf && lane == 0) atomicMax((unsigned long long*)&p.tbuf[(size_t)blockIdx.x * 8 + 2], (unsigned long long)wall_clock64());
+#endif
+    return;
+  }
   if (is_row_wave) {
-    // ---- row waves: gate (or given activation) -> decision -> up -> publish ------------------------------------
+    // ---- row waves: gate -> decision -> up -> publish ------------------------------------------------------------
     // A wave holds its current neuron, the next one (whose first gate block it prefetches) and the ticket after that.
     int cur = neuron_of(rw);
     int nxt = neuron_of(rw + RW);
     u32x4 wc[CB];
     stage([&] {
-      const u32x4* src = (gate && cur >= 0) ? p.wg + (size_t)cur * p.row_vecs : p.x;
+      const u32x4* src = cur >= 0 ? p.wg + (size_t)cur * p.row_vecs : p.x;
       fused_issue<CB, FULL>(src, 0, vlast, lane, wc);
     });
     const int nblk = nchp / CB;
-    const st* ain = (const st*)p.a_in;
     while (cur >= 0) {
       int pend = 0;
       if (lane == 0) pend = __hip_atomic_fetch_add(&s_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -289,7 +385,7 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       float a[B];
       bool act[B];
       bool any = false;
-      if (gate) {
+      {
         float g[B];
 #pragma unroll
         for (int b = 0; b < B; b++) g[b] = 0.f;
@@ -310,15 +406,6 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
           act[b] = b < p.nb && fabsf(a[b]) > p.t;
           any = any || act[b];
         }
-      } else {
-#pragma unroll
-        for (int b = 0; b < B; b++) {
-          const float av = b < p.nb ? DT::tof(ain[(size_t)b * p.I + row]) : 0.f;
-          act[b] = b < p.nb && fabsf(av) > p.t;
-          a[b] = av;
-          any = any || act[b];
-        }
-        any = __builtin_amdgcn_readfirstlane((int)any) != 0;
       }
       float z[B];
 #pragma unroll
@@ -362,7 +449,17 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   }
 
   // ---- down waves: walk the slots in neuron order, stream this wave's columns of every live neuron ----------------
-  stage([] {});
+  stage([&] {
+    if (!gate) {
+      // given activations: (nb, I) in dtype -> the z slots of this workgroup's neurons, as fp32 (exact); the row waves read
+      // them from there and overwrite them with z
+      const st* ain = (const st*)p.a_in;
+      for (int i = tid; i < n * B; i += kFusedDownWaves * kWave) {
+        const int q = i / B, b = i - q * B;
+        sl.z[i] = b < p.nb ? DT::tof(ain[(size_t)b * p.I + row0 + q]) : 0.f;
+      }
+    }
+  });
   const int d = wave;
   int vidx[KV];
 #pragma unroll
