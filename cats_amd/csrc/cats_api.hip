@@ -277,14 +277,15 @@ bool fused_eligible(int B, int H, int I, int dtype, FusedArgs& f, int& grid) {
   f.H = H; f.I = I; f.nb = B;
   f.row_vecs = H / vec;
   f.nch = (f.row_vecs + kWave - 1) / kWave;
-  if (f.row_vecs > kFusedMaxKV * kFusedDownWaves * kWave) return false;
+  const int bt = batch_template(B);
+  const int dw = fused_down_waves(bt), rw = kFusedWaves - dw;
+  if (f.row_vecs > kFusedMaxKV * dw * kWave) return false;
   int maxgrid = device_cus();
   if (maxgrid > kFusedMaxGrid) maxgrid = kFusedMaxGrid;
   int rpw = (I + maxgrid - 1) / maxgrid;
-  if (rpw < 2 * kFusedRowWaves) rpw = 2 * kFusedRowWaves;  // small matrices: fewer workgroups rather than idle row waves
+  if (rpw < 2 * rw) rpw = 2 * rw;  // small matrices: fewer workgroups rather than idle row waves
   grid = (I + rpw - 1) / rpw;
   f.rpw = rpw;
-  const int bt = batch_template(B);
   const size_t nchv = (size_t)(f.nch + kFusedCB - 1) / kFusedCB * kFusedCB * kWave;
   const size_t lds = bt * nchv * 16 + (size_t)((rpw + 3) & ~3) * 4 + (size_t)rpw * bt * 4;
   return lds <= 128 * 1024;

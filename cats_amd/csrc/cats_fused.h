@@ -1,9 +1,10 @@
 // Whole CATS MLP in one streaming launch plus a small reduction launch, for 1 or 2 batch rows.
 //
-//   mlp_fused_kernel   One persistent workgroup of 16 waves per CU owns a contiguous range of neurons.  Eight "row
-//                      waves" take the range's neurons one at a time (LDS ticket): gate row -> SiLU -> threshold, and
+//   mlp_fused_kernel   One persistent workgroup of 16 waves per CU owns a contiguous range of neurons.  Its "row
+//                      waves" (twelve at one batch row, eight at two) take the range's neurons one at a time (LDS
+//                      ticket): gate row -> SiLU -> threshold, and
 //                      for an active neuron the matching W_up row -> z.  The result of every neuron is published in an
-//                      LDS slot (dead, or live with its z).  Eight "down waves" own an eighth of the output columns
+//                      LDS slot (dead, or live with its z).  The other "down waves" own an equal part of the output columns
 //                      each; they walk the slots in neuron order and, for every live one, stream their part of that
 //                      neuron's W_down^T row into fp32 accumulators.  Nothing crosses a workgroup boundary while the
 //                      weights stream: no mask or z round trip through memory, no arrival counters, no second launch
@@ -26,11 +27,14 @@
 namespace cats {
 
 constexpr int kFusedWaves = 16;
-constexpr int kFusedDownWaves = 8;
-constexpr int kFusedRowWaves = kFusedWaves - kFusedDownWaves;
+// How the 16 waves split into down waves (each owns 1 / DW of the output columns) and row waves.  A row wave keeps one
+// gate row and one up row in flight and waits out a memory round trip per neuron, so at one batch row twelve of them
+// keep the machine busier than eight (measured: 34.6 against 35.5 us on the Llama layer); at two batch rows the down
+// waves carry twice the arithmetic per fetched row and four of them fall behind (45.6 against 42.6 us).
+constexpr int fused_down_waves(int batch_template) { return batch_template == 1 ? 4 : 8; }
 constexpr int kFusedThreads = kFusedWaves * kWave;
 constexpr int kFusedCB = 8;             // 64-lane chunks (of 16 bytes per lane) per block of row loads
-constexpr int kFusedMaxKV = 4;          // a down wave covers KV * 64 vectors of a row: rows of up to 4 * 8 * 64 vectors
+constexpr int kFusedMaxKV = 4;          // a down wave covers KV * 64 vectors of a row: rows of up to 4 * DW * 64 vectors
 constexpr int kReduceCols = 32;         // fp32 columns per workgroup of the reduction kernel
 constexpr int kReduceLanes = 32;        // ranges of partials summed side by side per column
 
@@ -189,12 +193,12 @@ __device__ __forceinline__ void fused_down_consume(const DownBatch<B, KV, RB>& b
   }
 }
 
-template <class DT, int B, bool FULL, int KV>
+template <class DT, int B, bool FULL, int KV, int DW>
 __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   typedef typename DT::st st;
   constexpr int CB = kFusedCB;
   constexpr int VEC = DT::VEC;
-  constexpr int RW = kFusedRowWaves;
+  constexpr int RW = kFusedWaves - DW;
   constexpr int RB = 8 / (KV * B) < 1 ? 1 : 8 / (KV * B);  // row slots per batch of a down wave; two batches are in flight
   constexpr int kXPre = 2;  // x vectors per thread fetched ahead of the first weight block
   extern __shared__ u32x4 s_fused[];
@@ -218,8 +222,8 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   sl.n = n;
 
   CATS_FSTAMP(tid == 0, 0);
-  const bool is_row_wave = wave >= kFusedDownWaves;
-  const int rw = wave - kFusedDownWaves;
+  const bool is_row_wave = wave >= DW;
+  const int rw = wave - DW;
   const bool gate = p.wg != nullptr;
 
   // Position in the workgroup's range -> neuron, or -1 past the end.
@@ -454,7 +458,7 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       // given activations: (nb, I) in dtype -> the z slots of this workgroup's neurons, as fp32 (exact); the row waves read
       // them from there and overwrite them with z
       const st* ain = (const st*)p.a_in;
-      for (int i = tid; i < n * B; i += kFusedDownWaves * kWave) {
+      for (int i = tid; i < n * B; i += DW * kWave) {
         const int q = i / B, b = i - q * B;
         sl.z[i] = b < p.nb ? DT::tof(ain[(size_t)b * p.I + row0 + q]) : 0.f;
       }
@@ -463,7 +467,7 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   const int d = wave;
   int vidx[KV];
 #pragma unroll
-  for (int k = 0; k < KV; k++) vidx[k] = min((k * kFusedDownWaves + d) * kWave + lane, vlast);
+  for (int k = 0; k < KV; k++) vidx[k] = min((k * DW + d) * kWave + lane, vlast);
   float acc[B][KV][VEC];
 #pragma unroll
   for (int b = 0; b < B; b++)
@@ -493,7 +497,7 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   float* mypart = p.partial + (size_t)blockIdx.x * p.nb * p.H;
 #pragma unroll
   for (int k = 0; k < KV; k++) {
-    const int v = (k * kFusedDownWaves + d) * kWave + lane;
+    const int v = (k * DW + d) * kWave + lane;
     if (v < p.row_vecs) {
 #pragma unroll
       for (int b = 0; b < B; b++)

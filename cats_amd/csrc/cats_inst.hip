@@ -130,9 +130,9 @@ hipError_t launch_down_one(const DownArgs& a, int block, hipStream_t stream) {
   return hipGetLastError();
 }
 
-template <class DT, int B, bool FULL, int KV>
+template <class DT, int B, bool FULL, int KV, int DW>
 hipError_t launch_fused_one(int grid, const FusedArgs& a, hipStream_t stream) {
-  auto kern = mlp_fused_kernel<DT, B, FULL, KV>;
+  auto kern = mlp_fused_kernel<DT, B, FULL, KV, DW>;
   const int nchv = (a.nch + kFusedCB - 1) / kFusedCB * kFusedCB * kWave;
   const size_t lds = (size_t)B * nchv * sizeof(u32x4) + (size_t)((a.rpw + 3) & ~3) * 4 + (size_t)a.rpw * B * 4;
   if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
@@ -143,10 +143,11 @@ hipError_t launch_fused_one(int grid, const FusedArgs& a, hipStream_t stream) {
 template <class DT, int B>
 hipError_t launch_fused_b(int grid, const FusedArgs& a, hipStream_t stream) {
   const bool full = a.H % (kWave * DT::VEC * kFusedCB) == 0;
-  const int kv = (a.row_vecs + kFusedDownWaves * kWave - 1) / (kFusedDownWaves * kWave);
-#define CATS_FUSED_KV(KVV)                                                              \
-  if (kv <= KVV) return full ? launch_fused_one<DT, B, true, KVV>(grid, a, stream)      \
-                             : launch_fused_one<DT, B, false, KVV>(grid, a, stream);
+  constexpr int DW = fused_down_waves(B);
+  const int kv = (a.row_vecs + DW * kWave - 1) / (DW * kWave);
+#define CATS_FUSED_KV(KVV)                                                                \
+  if (kv <= KVV) return full ? launch_fused_one<DT, B, true, KVV, DW>(grid, a, stream)    \
+                             : launch_fused_one<DT, B, false, KVV, DW>(grid, a, stream);
   CATS_FUSED_KV(1)
   CATS_FUSED_KV(2)
   CATS_FUSED_KV(4)

@@ -89,10 +89,12 @@ def main() -> None:
     med = torch.stack([r[:, 4].median() for r in rows])
     print(f"per call: last workgroup stored at {float(last.mean()):.2f} us (mean over calls), the median workgroup at "
           f"{float(med.mean()):.2f} us")
-    end, live = allr[:, 3], allr[:, 5]
-    c = torch.corrcoef(torch.stack([end, live]))[0, 1].item()
-    slope = float(((end - end.mean()) * (live - live.mean())).sum() / ((live - live.mean()) ** 2).sum())
-    print(f"end of the down pass against live neurons of the workgroup: correlation {c:.2f}, {slope:.3f} us per live neuron")
+    live = allr[:, 5]
+    for k, name in ((2, "last neuron published"), (3, "end of the down pass")):
+        end = allr[:, k]
+        c = torch.corrcoef(torch.stack([end, live]))[0, 1].item()
+        slope = float(((end - end.mean()) * (live - live.mean())).sum() / ((live - live.mean()) ** 2).sum())
+        print(f"{name} against live neurons of the workgroup: correlation {c:.2f}, {slope:.3f} us per live neuron")
     xcd = torch.arange(rows[0].shape[0]) % 8
     per_xcd = [float(torch.stack([r[xcd == k, 3].mean() for r in rows]).mean()) for k in range(8)]
     print("mean end of the down pass by blockIdx % 8 (workgroups are dealt round-robin over the 8 XCDs): "
