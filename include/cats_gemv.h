@@ -174,8 +174,8 @@ int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, co
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose ops
  * cudaMalloc per call).  The scratch of the single-pass kernels (per-workgroup partial sums and counts, 8 MiB + 4 KiB)
  * lives in a device array inside the library, one copy per GPU, held until the process ends; nothing is allocated or
- * freed by the call.  Limits: 1..2 rows, B * H <= 8192, rows of at most 2048 16-byte vectors; anything else returns
- * CATS_ERR_SCRATCH.  Same kernels and summation order as cats_mlp, so the same bits.  All calls on one GPU share
+ * freed by the call.  Limits: 1..2 rows, B * H <= 8192, rows of at most 1024 (one row) or 2048 (two rows) 16-byte
+ * vectors (fp32 at one row: H <= 4096); anything else returns CATS_ERR_SCRATCH.  Same kernels and summation order as cats_mlp, so the same bits.  All calls on one GPU share
  * that GPU's array: calls that overlap in time on one GPU (different streams, or a graph replay next to an eager
  * call) race; calls on one stream, or otherwise ordered, are fine.  Nothing in the array has to be cleared between
  * calls (every call overwrites what it reads). */
