@@ -27,6 +27,19 @@ template <> hipError_t launch_down<F32>(int, bool, const DownArgs&, int, hipStre
 template <> hipError_t launch_fused<F16>(int, int, int, const FusedArgs&, const ReduceArgs&, hipStream_t);
 template <> hipError_t launch_fused<BF16>(int, int, int, const FusedArgs&, const ReduceArgs&, hipStream_t);
 template <> hipError_t launch_fused<F32>(int, int, int, const FusedArgs&, const ReduceArgs&, hipStream_t);
+int current_device_cus() {
+  constexpr int kDevs = 64;
+  static int cus[kDevs];  // 0 = not asked yet; written once per device with the same value, so a plain atomic will do
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kDevs) return 256;
+  int n = __atomic_load_n(&cus[dev], __ATOMIC_RELAXED);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    __atomic_store_n(&cus[dev], n, __ATOMIC_RELAXED);
+  }
+  return n;
+}
+
 namespace {
 
 Tuning g_tuning = {0, 0, 0, 0};
@@ -256,22 +269,14 @@ int check_ws(const void* ws, size_t ws_bytes, int H, int I, WsLayout& l) {
   return CATS_OK;
 }
 
-int device_cus() {
-  static int cus = 0;  // every GPU of a node is the same part, so one query serves all
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cus = n;
-  }
-  return cus;
-}
 
 constexpr int kFusedMaxGrid = 256;  // partials of 256 workgroups x 2 batch rows fit the workspace's partial-sum region
 
 // Whether the single-pass kernel covers this call, and with what launch shape: one workgroup per CU, each with an
 // equal, contiguous share of the neurons.
-bool fused_eligible(int B, int H, int I, int dtype, FusedArgs& f, int& grid) {
-  if (g_tuning.path == 1 || B > 2) return false;
+// `any_path`: ignore the A/B knob that keeps whole-MLP calls on the separate kernels (cats_set_tuning(path = 1)).
+bool fused_eligible(int B, int H, int I, int dtype, FusedArgs& f, int& grid, bool any_path = false) {
+  if ((g_tuning.path == 1 && !any_path) || B > 2) return false;
   const int vec = vec_elems(dtype);
   memset(&f, 0, sizeof(f));
   f.H = H; f.I = I; f.nb = B;
@@ -280,21 +285,22 @@ bool fused_eligible(int B, int H, int I, int dtype, FusedArgs& f, int& grid) {
   const int bt = batch_template(B);
   const int dw = fused_down_waves(bt), rw = kFusedWaves - dw;
   if (f.row_vecs > kFusedMaxKV * dw * kWave) return false;
-  int maxgrid = device_cus();
+  int maxgrid = current_device_cus();
   if (maxgrid > kFusedMaxGrid) maxgrid = kFusedMaxGrid;
   int rpw = (I + maxgrid - 1) / maxgrid;
   if (rpw < 2 * rw) rpw = 2 * rw;  // small matrices: fewer workgroups rather than idle row waves
   grid = (I + rpw - 1) / rpw;
   f.rpw = rpw;
-  const size_t nchv = (size_t)(f.nch + kFusedCB - 1) / kFusedCB * kFusedCB * kWave;
-  const size_t lds = bt * nchv * 16 + (size_t)((rpw + 3) & ~3) * 4 + (size_t)rpw * bt * 4;
-  return lds <= 128 * 1024;
+  return fused_lds_bytes(bt, f.nch, rpw, vec, dw) <= 128 * 1024;
 }
 
+// y32 set: the streaming kernel adds into the caller's fp32 accumulator itself and nothing is launched after it,
+// unless the caller wants the count of active neurons (then the second launch does only that).
 int do_fused(FusedArgs& f, int grid, int stage, void* y_out, const void* residual, int32_t* count_out, int dtype, char* ws,
-             const WsLayout& l, hipStream_t s) {
+             const WsLayout& l, hipStream_t s, float* y32 = nullptr) {
   f.partial = (float*)(ws + l.partial);
   f.counts = (int32_t*)(ws + l.z32);
+  f.y32 = y32;
 #ifdef CATS_TIMING
   f.tbuf = g_tbuf_fused;
 #endif
@@ -308,6 +314,10 @@ int do_fused(FusedArgs& f, int grid, int stage, void* y_out, const void* residua
   r.H = f.H;
   r.G = grid;
   r.BH = f.nb * f.H;
+  if (y32) {
+    r.BH = 0;  // no columns to finish
+    if (stage == 0 && !count_out) stage = 1;
+  }
   const int bt = batch_template(f.nb);
   hipError_t e;
   if (dtype == CATS_F16) e = launch_fused<F16>(bt, grid, stage, f, r, s);
@@ -518,14 +528,14 @@ static int mlp_pass(const void* x, const void* wgate, const void* wup, const voi
   if (st) return st;
   FusedArgs f;
   int grid = 0;
-  if (y_out && fused_eligible(B, H, I, dtype, f, grid)) {
+  if (fused_eligible(B, H, I, dtype, f, grid)) {
     f.x = (const u32x4*)x;
     f.wg = (const u32x4*)wgate;
     f.wu = (const u32x4*)wup;
     f.wd = (const u32x4*)wdown_t;
     f.flag_out = flag_out;
     f.t = round_through(dtype, threshold);
-    return do_fused(f, grid, stage, y_out, nullptr, count_out, dtype, (char*)ws, l, (hipStream_t)stream);
+    return do_fused(f, grid, stage, y_out, nullptr, count_out, dtype, (char*)ws, l, (hipStream_t)stream, y_f32);
   }
   RowsArgs a;
   fill_rows(a, x, wgate, H, I, B, dtype);
@@ -762,10 +772,7 @@ int cats_mlp_noalloc(const void* x, const void* wgate, const void* wup, const vo
   if (!aligned16(x) || !aligned16(wgate) || !aligned16(wup) || !aligned16(wdown_t)) return CATS_ERR_ALIGN;
   FusedArgs f;
   int grid = 0;
-  const int saved_path = g_tuning.path;
-  g_tuning.path = 0;  // this entry point is the single-pass kernel or nothing
-  const bool ok = fused_eligible(B, H, I, dtype, f, grid);
-  g_tuning.path = saved_path;
+  const bool ok = fused_eligible(B, H, I, dtype, f, grid, true);  // this entry point is the single-pass kernel or nothing
   // the stated limit (B * H <= 8192) whatever the grid turns out to be, and the actual footprint as a second check
   if (!ok || (size_t)B * H > 8192 || (size_t)grid * B * H * 4 > kScratchPartialBytes || (size_t)grid * 4 > kScratchBytes - kScratchPartialBytes)
     return CATS_ERR_SCRATCH;

@@ -38,7 +38,18 @@ constexpr int kFusedMaxKV = 4;          // a down wave covers KV * 64 vectors of
 constexpr int kReduceCols = 32;         // fp32 columns per workgroup of the reduction kernel
 constexpr int kReduceLanes = 32;        // ranges of partials summed side by side per column
 
-enum FusedSlot { kSlotPending = 0, kSlotDead = 1, kSlotLive = 2 };
+// Pending: not decided yet.  Dead: no batch row keeps the neuron.  Announced: some row keeps it, its z is still being
+// computed -- enough for a down wave to send for the neuron's W_down^T row.  Live: z is in the slot.
+// Dynamic LDS of mlp_fused_kernel: the staged x rows, the slot states, the slot z values, and one area per down wave in
+// which it regroups its sums by column before the atomics of the y32 mode.  bt: compile-time batch, vec: elements per
+// 16-byte vector, dw: down waves.
+inline size_t fused_lds_bytes(int bt, int nch, int rpw, int vec, int dw) {
+  const size_t nchv = (size_t)(nch + kFusedCB - 1) / kFusedCB * kFusedCB * kWave;
+  return (size_t)bt * nchv * 16 + (size_t)((rpw + 3) & ~3) * 4 + (size_t)((rpw * bt + 3) & ~3) * 4 + (size_t)dw * kWave * vec * 4;
+}
+
+enum FusedSlot { kSlotPending = 0, kSlotDead = 1, kSlotAnnounced = 2, kSlotLive = 3 };
+
 
 struct FusedArgs {
   const u32x4* x;        // (nb, H)
@@ -48,6 +59,7 @@ struct FusedArgs {
   const void* a_in;      // optional (nb, I) dtype: gate activations; flags = |a| > t
   uint8_t* flag_out;     // optional (nb, I)
   float* partial;        // [grid][nb][H] fp32
+  float* y32;            // optional (nb, H) fp32: the workgroup adds its sums here with atomics instead of storing `partial`
   int32_t* counts;       // [grid] live neurons per workgroup
   const u32x4* norm_w;   // optional (H,) RMS-norm weight applied to x while it is staged
   float norm_eps;
@@ -108,6 +120,7 @@ struct DownBatch {
   int rows[RB];       // neuron index, -1 = empty slot
   float zz[RB][B];
   int cnt;
+  int unresolved;     // bit u: row u was taken while only announced, its z is still to be fetched
   u32x4 wv[RB][KV];
 };
 
@@ -118,13 +131,16 @@ struct FusedSlots {
   int row0, n;
 };
 
-// Fill the batch with the next live neurons whose slots are published, in neuron order.  Blocking: wait until at
-// least one is there or the range is exhausted.  Non-blocking: take what is there, possibly nothing.
+// Fill the batch with the next neurons that some batch row keeps, in neuron order, as far as the slots are decided.
+// Announced is enough to take a neuron: its row can be sent for, and fused_resolve fetches its z later; the z of a slot
+// that is already live is taken here.  Blocking: wait until at least one is there or the range is exhausted.
+// Non-blocking: take what is there, possibly nothing.
 // The wave looks at 64 slots per pass -- lane i reads state and z of slot head + i, ballots find the decided prefix and
-// the live slots in it -- so a pass costs one LDS round trip however many dead slots it steps over.
+// the kept slots in it -- so a pass costs one LDS round trip however many dead slots it steps over.
 template <int B, int KV, int RB>
 __device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const FusedSlots& sl, int& head, bool blocking) {
   bt.cnt = 0;
+  bt.unresolved = 0;
 #pragma unroll
   for (int u = 0; u < RB; u++) {
     bt.rows[u] = -1;
@@ -138,14 +154,15 @@ __device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const Fu
     // past the end counts as pending: it ends the decided prefix
     const int st_ = in ? __hip_atomic_load(&sl.state[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : kSlotPending;
     const uint64_t pend = __ballot(st_ == kSlotPending);
-    uint64_t live = __ballot(st_ == kSlotLive);
+    uint64_t live = __ballot(st_ >= kSlotAnnounced);
+    const uint64_t hasz = __ballot(st_ == kSlotLive);
     const int ready = pend ? __builtin_ctzll(pend) : kWave;  // slots head .. head + ready - 1 are decided
     if (ready == 0) {
       if (!blocking) return;
       __builtin_amdgcn_s_sleep(1);
       continue;
     }
-    // acquire side of the hand-off (LDS only): the z of every slot seen decided above is read after its state
+    // acquire side of the hand-off (LDS only): the z of every slot seen live above is read after its state
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     int zv[B];
 #pragma unroll
@@ -157,15 +174,49 @@ __device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const Fu
         const int bit = __builtin_ctzll(live);
         live &= live - 1ull;
         bt.rows[u] = sl.row0 + head + bit;
+        if ((hasz >> bit) & 1ull) {
 #pragma unroll
-        for (int b = 0; b < B; b++) bt.zz[u][b] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zv[b], bit));
+          for (int b = 0; b < B; b++) bt.zz[u][b] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zv[b], bit));
+        } else {
+          bt.unresolved |= 1 << u;
+        }
         bt.cnt++;
       }
     }
-    head += live ? __builtin_ctzll(live) : ready;  // up to the first live slot that did not fit, else past the decided prefix
+    head += live ? __builtin_ctzll(live) : ready;  // up to the first kept slot that did not fit, else past the decided prefix
     if (bt.cnt > 0) return;
     // only dead slots so far: keep going
   }
+}
+
+// Wait until the z of every row of the batch is in its slot, and read those that fused_collect could not.  Lane u
+// watches row u.
+template <int B, int KV, int RB>
+__device__ __forceinline__ void fused_resolve(DownBatch<B, KV, RB>& bt, const FusedSlots& sl) {
+  if (bt.unresolved == 0) return;  // uniform
+  const int lane = threadIdx.x & (kWave - 1);
+  int myslot = -1;
+#pragma unroll
+  for (int u = 0; u < RB; u++)
+    if (lane == u && ((bt.unresolved >> u) & 1)) myslot = bt.rows[u] - sl.row0;
+  for (;;) {
+    const int st_ = myslot >= 0 ? __hip_atomic_load(&sl.state[myslot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : kSlotLive;
+    if (__ballot(st_ != kSlotLive) == 0ull) break;
+    __builtin_amdgcn_s_sleep(1);
+  }
+  // acquire side of the hand-off (LDS only): the z of every slot seen live above is read after its state
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+  int zv[B];
+#pragma unroll
+  for (int b = 0; b < B; b++) zv[b] = myslot >= 0 ? __builtin_bit_cast(int, sl.z[myslot * B + b]) : 0;
+#pragma unroll
+  for (int u = 0; u < RB; u++) {
+    if ((bt.unresolved >> u) & 1) {  // uniform
+#pragma unroll
+      for (int b = 0; b < B; b++) bt.zz[u][b] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zv[b], u));
+    }
+  }
+  bt.unresolved = 0;
 }
 
 template <int B, int KV, int RB>
@@ -220,6 +271,7 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   sl.z = (float*)(sl.state + ((p.rpw + 3) & ~3));  // [rpw][B]
   sl.row0 = row0;
   sl.n = n;
+  float* tr_all = sl.z + ((p.rpw * B + 3) & ~3);   // [DW][64 * VEC]: where a down wave regroups its sums by column (y32 mode)
 
   CATS_FSTAMP(tid == 0, 0);
   const bool is_row_wave = wave >= DW;
@@ -253,7 +305,9 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       if (b < p.nb && v < p.row_vecs) val = p.x[(size_t)b * p.row_vecs + v];
       xs[i] = val;
     }
-    for (int i = tid; i < p.rpw; i += kFusedThreads) sl.state[i] = kSlotPending;
+    // given activations: the down waves decide every slot (announced or dead) while they stage the activations
+    if (gate)
+      for (int i = tid; i < p.rpw; i += kFusedThreads) sl.state[i] = kSlotPending;
     // gate mode: the first two neurons of every row wave are fixed, the rest go by ticket; given activations: all by ticket
     if (tid == 0) s_ticket = gate ? 2 * RW : 0;
     __syncthreads();
@@ -276,9 +330,9 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   };
 
   if (is_row_wave && !gate) {
-    // ---- row waves, gate activations given: the down waves have put them into the z slots while x was staged, so a
-    // wave knows whether a neuron is live from one LDS read.  It walks its tickets, publishes dead neurons at once and
-    // keeps the up rows of two live neurons (in blocks of CB chunks) in flight: the block of the next unit goes out
+    // ---- row waves, gate activations given: the down waves have put them into the z slots while x was staged (and
+    // marked every slot announced or dead), so a wave knows whether a neuron is live from one LDS read.  It walks its
+    // tickets and keeps the up rows of two live neurons (in blocks of CB chunks) in flight: the block of the next unit goes out
     // before the current one is multiplied, both buffers always take a full block of loads (x, cached, when there is
     // nothing left) so the wait for the older one is a fixed count.
     stage([] {});
@@ -305,13 +359,7 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
           for (int b = 0; b < B; b++)
             if (b < p.nb) p.flag_out[(size_t)b * p.I + row0 + q] = iact[b] ? 1 : 0;
         }
-        if (any) return row0 + q;
-        if (lane == 0) {
-#pragma unroll
-          for (int b = 0; b < B; b++) sl.z[q * B + b] = 0.f;
-          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-          __hip_atomic_store(&sl.state[q], kSlotDead, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        }
+        if (any) return row0 + q;  // a dead neuron's slot already says so
       }
     };
     // one unit = one block of one live neuron's up row; row < 0 = nothing left (the loads still go out, to x)
@@ -414,7 +462,12 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       float z[B];
 #pragma unroll
       for (int b = 0; b < B; b++) z[b] = 0.f;
+#ifdef CATS_TIMING
+      if (p.tbuf && lane == 0) atomicMax((unsigned long long*)&p.tbuf[(size_t)blockIdx.x * 8 + 7], (unsigned long long)wall_clock64());
+#endif
       if (any) {  // wave-uniform
+        // the down waves may send for this neuron's W_down^T row now: it travels while the W_up row does
+        if (lane == 0) __hip_atomic_store(&sl.state[row - row0], kSlotAnnounced, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         float u[B];
 #pragma unroll
         for (int b = 0; b < B; b++) u[b] = 0.f;
@@ -458,9 +511,15 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       // given activations: (nb, I) in dtype -> the z slots of this workgroup's neurons, as fp32 (exact); the row waves read
       // them from there and overwrite them with z
       const st* ain = (const st*)p.a_in;
-      for (int i = tid; i < n * B; i += DW * kWave) {
-        const int q = i / B, b = i - q * B;
-        sl.z[i] = b < p.nb ? DT::tof(ain[(size_t)b * p.I + row0 + q]) : 0.f;
+      for (int q = tid; q < n; q += DW * kWave) {
+        bool any = false;
+#pragma unroll
+        for (int b = 0; b < B; b++) {
+          const float av = b < p.nb ? DT::tof(ain[(size_t)b * p.I + row0 + q]) : 0.f;
+          sl.z[q * B + b] = av;
+          any = any || (b < p.nb && fabsf(av) > p.t);
+        }
+        sl.state[q] = any ? kSlotAnnounced : kSlotDead;  // ordered before any reader by the staging barrier
       }
     }
   });
@@ -483,32 +542,92 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   for (;;) {
     if (ba.cnt == 0 && head >= n) break;
     fused_collect<B, KV, RB>(bb, sl, head, ba.cnt == 0);
+    if (bb.cnt == 0 && head >= n) {
+      // nothing left to send for: finish the batch in flight and leave no load behind (whatever is still outstanding
+      // when the sums are written out has to be waited for first)
+      fused_resolve<B, KV, RB>(ba, sl);
+      fused_down_consume<DT, B, KV, RB>(ba, acc);
+      nlive += ba.cnt;
+      break;
+    }
+    CATS_FSTAMP(lane == 0 && d == 0 && bb.cnt > 0, 5);
     fused_down_issue<B, KV, RB>(bb, p.wd, p.row_vecs, p.x, vidx);
+    fused_resolve<B, KV, RB>(ba, sl);
     fused_down_consume<DT, B, KV, RB>(ba, acc);
     nlive += ba.cnt;
-    if (bb.cnt == 0 && head >= n) break;
     fused_collect<B, KV, RB>(ba, sl, head, bb.cnt == 0);
+    if (ba.cnt == 0 && head >= n) {
+      fused_resolve<B, KV, RB>(bb, sl);
+      fused_down_consume<DT, B, KV, RB>(bb, acc);
+      nlive += bb.cnt;
+      break;
+    }
+    CATS_FSTAMP(lane == 0 && d == 0 && ba.cnt > 0, 5);
     fused_down_issue<B, KV, RB>(ba, p.wd, p.row_vecs, p.x, vidx);
+    fused_resolve<B, KV, RB>(bb, sl);
     fused_down_consume<DT, B, KV, RB>(bb, acc);
     nlive += bb.cnt;
   }
   CATS_FSTAMP(lane == 0 && d == 0, 3);
 
-  float* mypart = p.partial + (size_t)blockIdx.x * p.nb * p.H;
+  if (p.y32) {
+    // The caller's fp32 accumulator: one atomic per column per workgroup.  A lane's sums are VEC neighbouring columns;
+    // regrouped through a wave-private piece of LDS every atomic instruction covers 64 neighbouring columns (two whole
+    // cache lines).  The order in which a workgroup walks its column groups is rotated by its number, so the 256
+    // workgroups, which finish together, do not all queue on the same lines.
+    float* tr = tr_all + d * (kWave * VEC);
+    const int rot = blockIdx.x;
 #pragma unroll
-  for (int k = 0; k < KV; k++) {
-    const int v = (k * DW + d) * kWave + lane;
-    if (v < p.row_vecs) {
+    for (int kk = 0; kk < KV; kk++) {
 #pragma unroll
-      for (int b = 0; b < B; b++)
+      for (int b = 0; b < B; b++) {
         if (b < p.nb) {
-          float4* dst = (float4*)(mypart + (size_t)b * p.H + (size_t)v * VEC);
+          float4* trv = (float4*)(tr + lane * VEC);
 #pragma unroll
           for (int q = 0; q < VEC / 4; q++) {
-            float4 o = {acc[b][k][4 * q], acc[b][k][4 * q + 1], acc[b][k][4 * q + 2], acc[b][k][4 * q + 3]};
-            dst[q] = o;
+            // which of the wave's KV column blocks goes first is rotated as well (a register select, no indexing)
+            float4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int k = 0; k < KV; k++)
+              if (((kk + (rot / VEC)) % KV) == k) { o.x = acc[b][k][4 * q]; o.y = acc[b][k][4 * q + 1]; o.z = acc[b][k][4 * q + 2]; o.w = acc[b][k][4 * q + 3]; }
+            trv[q] = o;
           }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+          const int k = (kk + (rot / VEC)) % KV;
+          const int col0 = (k * DW + d) * kWave * VEC;
+          // all LDS reads of the round first (one wait), then the atomics back to back
+          float tv[VEC];
+#pragma unroll
+          for (int j = 0; j < VEC; j++) tv[j] = tr[((j + rot) % VEC) * kWave + lane];
+#pragma unroll
+          for (int j = 0; j < VEC; j++) {
+            const int col = col0 + ((j + rot) % VEC) * kWave + lane;
+            if (col < p.H) unsafeAtomicAdd(p.y32 + (size_t)b * p.H + col, tv[j]);
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+          __builtin_amdgcn_wave_barrier();  // the next round overwrites tr
         }
+      }
+    }
+  } else {
+    float* mypart = p.partial + (size_t)blockIdx.x * p.nb * p.H;
+#pragma unroll
+    for (int k = 0; k < KV; k++) {
+      const int v = (k * DW + d) * kWave + lane;
+      if (v < p.row_vecs) {
+#pragma unroll
+        for (int b = 0; b < B; b++)
+          if (b < p.nb) {
+            float4* dst = (float4*)(mypart + (size_t)b * p.H + (size_t)v * VEC);
+#pragma unroll
+            for (int q = 0; q < VEC / 4; q++) {
+              float4 o = {acc[b][k][4 * q], acc[b][k][4 * q + 1], acc[b][k][4 * q + 2], acc[b][k][4 * q + 3]};
+              dst[q] = o;
+            }
+          }
+      }
     }
   }
   if (d == 0 && lane == 0) p.counts[blockIdx.x] = nlive;

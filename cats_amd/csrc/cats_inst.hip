@@ -64,12 +64,7 @@ struct MmaLaunch16 {
     return (steps == 4 || steps == 8) && rows_mma_lds_bytes(a.K) <= 160 * 1024;
   }
   static hipError_t run(const RowsArgs& a, bool up, hipStream_t stream) {
-    static int cus = 0;  // one workgroup per CU; every GPU of a node is the same part, so one query serves all
-    if (cus == 0) {
-      int dev = 0, n = 0;
-      if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-      cus = n;
-    }
+    const int cus = current_device_cus();  // one workgroup per CU
     const bool s8 = rows_mma_steps(a.K) == 8;
     auto kern = up ? (s8 ? rows_mma_kernel<DT, 8, true> : rows_mma_kernel<DT, 4, true>)
                    : (s8 ? rows_mma_kernel<DT, 8, false> : rows_mma_kernel<DT, 4, false>);
@@ -133,8 +128,7 @@ hipError_t launch_down_one(const DownArgs& a, int block, hipStream_t stream) {
 template <class DT, int B, bool FULL, int KV, int DW>
 hipError_t launch_fused_one(int grid, const FusedArgs& a, hipStream_t stream) {
   auto kern = mlp_fused_kernel<DT, B, FULL, KV, DW>;
-  const int nchv = (a.nch + kFusedCB - 1) / kFusedCB * kFusedCB * kWave;
-  const size_t lds = (size_t)B * nchv * sizeof(u32x4) + (size_t)((a.rpw + 3) & ~3) * 4 + (size_t)a.rpw * B * 4;
+  const size_t lds = fused_lds_bytes(B, a.nch, a.rpw, DT::VEC, DW);
   if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kFusedThreads), lds, stream, a);
   return hipGetLastError();
@@ -164,7 +158,8 @@ hipError_t launch_fused<CATS_DT>(int bt, int grid, int stage, const FusedArgs& a
     if (e != hipSuccess) return e;
   }
   if (stage != 1) {
-    hipLaunchKernelGGL(reduce_partials_kernel<CATS_DT>, dim3((r.BH + kReduceCols - 1) / kReduceCols), dim3(256), 0, stream, r);
+    const int rgrid = (r.BH + kReduceCols - 1) / kReduceCols;  // BH == 0: only the count is wanted
+    hipLaunchKernelGGL(reduce_partials_kernel<CATS_DT>, dim3(rgrid > 0 ? rgrid : 1), dim3(256), 0, stream, r);
     return hipGetLastError();
   }
   return hipSuccess;

@@ -15,6 +15,9 @@ struct Tuning {
   int path;          // whole-MLP entry points: 0 = choose by shape, 1 = always the separate gate+up and down kernels
 };
 
+// Compute units of the current device (256 if the runtime will not say), remembered per device.
+int current_device_cus();
+
 // Returns hipSuccess or the launch error.  `mode` is a RowsMode; bt (1, 2, 4 or 8) the compile-time batch.
 template <class DT>
 hipError_t launch_rows(int mode, int bt, const RowsArgs& a, hipStream_t stream);

@@ -55,8 +55,14 @@ def check_mlp_case(oracle, m, t, *, tag, ws=None, expect_flip_free=False):
         with pytest.raises(capi.CatsError, match="aligned"):
             capi.mlp_rowmajor_down(d["x"], d["wg"], d["wu"], d["wd"], t, ws)
         y_rm = y
+    # fp32-accumulate contract (fuse_gemv_gemv_gemv, flag_gemv_gemv_atomic): the call adds onto what the buffer holds
+    y32 = torch.ones(B, H, dtype=torch.float32, device="cuda")
+    _, flag32, count32 = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True, y_f32=y32)
     torch.cuda.synchronize()
     a, flag, y, flag2, y_rm = a.cpu(), flag.cpu(), y.cpu(), flag2.cpu(), y_rm.cpu()
+    y32 = y32.cpu() - 1.0
+    assert torch.equal(flag32.cpu(), flag2), f"{tag}: fp32-accumulate call disagrees on flags"
+    assert int(count32.item()) == int(count.item()), f"{tag}: fp32-accumulate call disagrees on the active count"
 
     # 1. mask rule, bit-exact on identical gate values: torch's own comparison on the kernel's activations
     want_flag = torch.abs(a) > t
@@ -90,6 +96,7 @@ def check_mlp_case(oracle, m, t, *, tag, ws=None, expect_flip_free=False):
     ref_same = oracle.c_mlp(m["x"], m["wg"], m["wu"], m["wd"], t, a_in=a, flag_in=flag)
     close(y, ref_same["y"], dtype)
     close(y_rm, ref_same["y"], dtype)
+    close(y32, ref_same["y"], dtype)  # atomics: summation order varies run to run, hence the tolerance and not bits
     # 5. and vs the fully independent oracle / the literal PyTorch formula when no flag flipped
     if nflip == 0:
         close(y, ref["y"], dtype)
