@@ -12,7 +12,8 @@ Three shared objects come out of this:
   stamps the wall clock at its phase boundaries into a caller-supplied buffer.  Only ``cats_amd.phase_stamps``
   loads it.
 
-Run ``python -m cats_amd.build`` (hipcc cross-compiles for gfx950 without a GPU).
+Run ``python -m cats_amd.build`` (hipcc cross-compiles for gfx950 without a GPU); ``--timing`` also builds the
+stamped twin.  ``CATS_HIP_DEFINES`` in the environment adds compiler definitions to the kernel builds.
 """
 from __future__ import annotations
 
@@ -55,6 +56,7 @@ def build_kernels(jobs: int = 4, timing: bool = False) -> Path:
     obj = OBJ / "timing" if timing else OBJ
     out = TIMING_LIB if timing else KERNEL_LIB
     extra = ["-DCATS_TIMING"] if timing else []
+    extra += os.environ.get("CATS_HIP_DEFINES", "").split()  # experiment switches, e.g. -DCATS_FUSED_POOL=1
     obj.mkdir(parents=True, exist_ok=True)
     LIB_DIR.mkdir(parents=True, exist_ok=True)
     units = [
@@ -92,11 +94,13 @@ def build_torch_shim() -> Path:
     return TORCH_LIB
 
 
-def build_all() -> None:
+def build_all(timing: bool = False) -> None:
+    """The product: kernel library and torch op library.  ``timing`` adds the stamped twin (a measuring tool)."""
     print(f"[cats_amd.build] kernels  -> {build_kernels()}")
     print(f"[cats_amd.build] torch op -> {build_torch_shim()}")
-    print(f"[cats_amd.build] stamped  -> {build_kernels(timing=True)}")
+    if timing:
+        print(f"[cats_amd.build] stamped  -> {build_kernels(timing=True)}")
 
 
 if __name__ == "__main__":
-    build_all()
+    build_all(timing="--timing" in sys.argv[1:])

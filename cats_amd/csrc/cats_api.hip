@@ -12,7 +12,9 @@
 // Built-in scratch of cats_mlp_noalloc: the per-workgroup partial sums and active counts of the single-pass kernel.
 // Every GPU the library runs on holds its own copy of this array, at its own address, until the process ends.
 constexpr size_t kScratchPartialBytes = (size_t)256 * 8192 * 4;  // 256 workgroups x (B * H <= 8192) fp32 partial sums
-constexpr size_t kScratchBytes = kScratchPartialBytes + 4096;    // + one int32 count per workgroup
+constexpr size_t kScratchCountBytes = 4096;                      // one int32 count per workgroup
+constexpr size_t kScratchPoolBytes = 4096;                       // neuron-pool counters of 32 workgroup groups
+constexpr size_t kScratchBytes = kScratchPartialBytes + kScratchCountBytes + kScratchPoolBytes;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 namespace cats {
@@ -51,7 +53,13 @@ long long* g_tbuf_fused = nullptr;
 
 constexpr int kMaxSlabs = 128;
 constexpr int kKernelBatch = 8;  // rows one launch handles; the entry points take up to CATS_MAX_BATCH rows in passes of this many
-constexpr size_t kCounterBytes = 1024 + 64 * 128;  // reserved head of the workspace; no kernel keeps state in it any more
+// Head of the workspace: the neuron-pool counters of the single-pass kernel (one 128-byte line per group of workgroups).
+// Zeroed by cats_workspace_init and put back to zero by every call that uses them.
+constexpr size_t kCounterBytes = 1024 + 64 * 128;
+#ifndef CATS_POOL_NUM  // share of a workgroup's neurons that goes to its group's pool (builds with -DCATS_FUSED_POOL=1 only)
+#define CATS_POOL_NUM 1
+#define CATS_POOL_DEN 4
+#endif
 
 __global__ void fill_zero_kernel(u32x4* p, size_t n16) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) p[i] = zero4();
@@ -291,7 +299,25 @@ bool fused_eligible(int B, int H, int I, int dtype, FusedArgs& f, int& grid, boo
   if (rpw < 2 * rw) rpw = 2 * rw;  // small matrices: fewer workgroups rather than idle row waves
   grid = (I + rpw - 1) / rpw;
   f.rpw = rpw;
-  return fused_lds_bytes(bt, f.nch, rpw, vec, dw) <= 128 * 1024;
+  f.spw = rpw;
+  f.cap = rpw;
+  return fused_lds_bytes(bt, f.nch, f.cap, vec, dw) <= 128 * 1024;
+}
+
+// Give the call a neuron pool if its shape allows: a fixed fraction of every workgroup's neurons goes to the pool of
+// its group.  `counters`: pool counter lines, zero, at least kPoolStride int32 per group of kFusedGroup workgroups.
+void fused_enable_pool(FusedArgs& f, int grid, int dtype, int32_t* counters, size_t counter_bytes) {
+  if (!kFusedPool || !f.wg || CATS_POOL_NUM == 0) return;  // given activations: no gate rows to balance, shares stay fixed
+  const int bt = batch_template(f.nb);
+  const int dw = fused_down_waves(bt), rw = kFusedWaves - dw;
+  const int spw = f.rpw - f.rpw * CATS_POOL_NUM / CATS_POOL_DEN;
+  const int groups = (grid + kFusedGroup - 1) / kFusedGroup;
+  if (spw == f.rpw || spw < 2 * rw || (size_t)groups * kPoolStride * 4 > counter_bytes) return;
+  const int cap = fused_slot_cap(spw, f.rpw, rw, true);
+  if (fused_lds_bytes(bt, f.nch, cap, vec_elems(dtype), dw) > 128 * 1024) return;
+  f.spw = spw;
+  f.cap = cap;
+  f.pool = counters;
 }
 
 // y32 set: the streaming kernel adds into the caller's fp32 accumulator itself and nothing is launched after it,
@@ -301,6 +327,7 @@ int do_fused(FusedArgs& f, int grid, int stage, void* y_out, const void* residua
   f.partial = (float*)(ws + l.partial);
   f.counts = (int32_t*)(ws + l.z32);
   f.y32 = y32;
+  fused_enable_pool(f, grid, dtype, (int32_t*)(ws + l.counters), kCounterBytes);
 #ifdef CATS_TIMING
   f.tbuf = g_tbuf_fused;
 #endif
@@ -387,7 +414,7 @@ const char* cats_status_string(int status) {
     case CATS_ERR_NULL: return "required pointer is NULL";
     case CATS_ERR_WORKSPACE: return "workspace missing, misaligned (256 bytes) or smaller than cats_workspace_bytes()";
     case CATS_ERR_LAUNCH: return "HIP kernel launch failed";
-    case CATS_ERR_SCRATCH: return "call does not fit the built-in scratch of cats_mlp_noalloc (1..2 rows, B * H <= 8192, rows of at most 2048 16-byte vectors)";
+    case CATS_ERR_SCRATCH: return "call does not fit the built-in scratch of cats_mlp_noalloc (1..2 rows, B * H <= 8192, rows of at most 1024 16-byte vectors at 1 row and 2048 at 2 rows)";
   }
   return "unknown status";
 }
@@ -412,8 +439,7 @@ int cats_workspace_init(void* ws, size_t ws_bytes, void* stream) {
   int grid = (int)((n16 + 255) / 256);
   if (grid > 2048) grid = 2048;
   if (grid < 1) grid = 1;
-  hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (u32x4*)ws, n16);
-  return hipGetLastError() == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+  return launch_kernel(fill_zero_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (u32x4*)ws, n16) == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
 }
 
 static int gate_flag_pass(const void* x, const void* wgate, void* a_out, uint8_t* flag_out, int B, int H, int I, int dtype,
@@ -460,17 +486,26 @@ int cats_gate_compact(const void* x, const void* wgate, void* vals_out, int64_t*
   if (groups > 64) groups = 64;
   c.bytes_per_group = (nbytes + groups - 1) / groups;
   groups = (nbytes + c.bytes_per_group - 1) / c.bytes_per_group;  // the last group's range is never empty: it writes the count
-  if (elem_size(dtype) == 2) hipLaunchKernelGGL(compact_kernel<2>, dim3(groups), dim3(256), 0, (hipStream_t)stream, c);
-  else hipLaunchKernelGGL(compact_kernel<4>, dim3(groups), dim3(256), 0, (hipStream_t)stream, c);
-  return hipGetLastError() == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+  const hipError_t e = elem_size(dtype) == 2 ? launch_kernel(compact_kernel<2>, dim3(groups), dim3(256), 0, (hipStream_t)stream, c)
+                                             : launch_kernel(compact_kernel<4>, dim3(groups), dim3(256), 0, (hipStream_t)stream, c);
+  return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
 }
 
 int cats_read_count(const int32_t* count_dev, void* stream) {
+  // One asynchronous copy into pinned host memory behind the caller's work on the stream, then one wait for the stream.
+  // The pinned word is allocated on first use and shared, so readers take turns.
+  static std::mutex mu;
+  static int32_t* pinned = nullptr;
   if (!count_dev) return -1;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!pinned && hipHostMalloc((void**)&pinned, 64, hipHostMallocDefault) != hipSuccess) {
+    pinned = nullptr;
+    return -1;
+  }
+  *pinned = -1;
+  if (hipMemcpyAsync(pinned, count_dev, sizeof(int32_t), hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess) return -1;
   if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return -1;
-  int32_t v = -1;
-  if (hipMemcpy(&v, count_dev, sizeof(v), hipMemcpyDeviceToHost) != hipSuccess) return -1;
-  return v;
+  return *pinned;
 }
 
 static int up_flag_pass(const void* x, const void* wup, const void* a_in, const uint8_t* flag, void* out, int out_is_f32, int B,
@@ -703,8 +738,9 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
                     stream);
   });
   if (st || !union_count) return st;
-  union_count_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(flag_out, B, I, count_out);
-  return hipGetLastError() == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+  return launch_kernel(union_count_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const uint8_t*)flag_out, B, I, count_out) == hipSuccess
+             ? CATS_OK
+             : CATS_ERR_LAUNCH;
 }
 
 int cats_mlp_stage(int stage, const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,
@@ -774,7 +810,7 @@ int cats_mlp_noalloc(const void* x, const void* wgate, const void* wup, const vo
   int grid = 0;
   const bool ok = fused_eligible(B, H, I, dtype, f, grid, true);  // this entry point is the single-pass kernel or nothing
   // the stated limit (B * H <= 8192) whatever the grid turns out to be, and the actual footprint as a second check
-  if (!ok || (size_t)B * H > 8192 || (size_t)grid * B * H * 4 > kScratchPartialBytes || (size_t)grid * 4 > kScratchBytes - kScratchPartialBytes)
+  if (!ok || (size_t)B * H > 8192 || (size_t)grid * B * H * 4 > kScratchPartialBytes || (size_t)grid * 4 > kScratchCountBytes)
     return CATS_ERR_SCRATCH;
   void* sp = nullptr;
   st = scratch_address(&sp);
@@ -786,6 +822,7 @@ int cats_mlp_noalloc(const void* x, const void* wgate, const void* wup, const vo
   f.t = round_through(dtype, threshold);
   f.partial = (float*)sp;
   f.counts = (int32_t*)((char*)sp + kScratchPartialBytes);
+  fused_enable_pool(f, grid, dtype, (int32_t*)((char*)sp + kScratchPartialBytes + kScratchCountBytes), kScratchPoolBytes);
   ReduceArgs r;
   memset(&r, 0, sizeof(r));
   r.partial = f.partial;

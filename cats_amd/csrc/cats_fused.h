@@ -35,6 +35,15 @@ constexpr int fused_down_waves(int batch_template) { return batch_template == 1 
 constexpr int kFusedThreads = kFusedWaves * kWave;
 constexpr int kFusedCB = 8;             // 64-lane chunks (of 16 bytes per lane) per block of row loads
 constexpr int kFusedMaxKV = 4;          // a down wave covers KV * 64 vectors of a row: rows of up to 4 * DW * 64 vectors
+// Experiment switch, off in the product build: -DCATS_FUSED_POOL=1 compiles the neuron pool described at the kernel
+// (dynamic balancing between the workgroups of a group).  Measured slower than fixed shares on the MI355X, kept so the
+// measurement can be repeated.
+#ifndef CATS_FUSED_POOL
+#define CATS_FUSED_POOL 0
+#endif
+constexpr bool kFusedPool = CATS_FUSED_POOL != 0;
+constexpr int kFusedGroup = 8;          // consecutive workgroups (one per XCD) that share a pool of neurons
+constexpr int kPoolStride = 32;         // int32 per group in the pool counter array: ticket counter at +0, finished workgroups at +16
 constexpr int kReduceCols = 32;         // fp32 columns per workgroup of the reduction kernel
 constexpr int kReduceLanes = 32;        // ranges of partials summed side by side per column
 
@@ -43,9 +52,17 @@ constexpr int kReduceLanes = 32;        // ranges of partials summed side by sid
 // Dynamic LDS of mlp_fused_kernel: the staged x rows, the slot states, the slot z values, and one area per down wave in
 // which it regroups its sums by column before the atomics of the y32 mode.  bt: compile-time batch, vec: elements per
 // 16-byte vector, dw: down waves.
-inline size_t fused_lds_bytes(int bt, int nch, int rpw, int vec, int dw) {
+// cap: slots per workgroup (fused_slot_cap).
+inline size_t fused_lds_bytes(int bt, int nch, int cap, int vec, int dw) {
   const size_t nchv = (size_t)(nch + kFusedCB - 1) / kFusedCB * kFusedCB * kWave;
-  return (size_t)bt * nchv * 16 + (size_t)((rpw + 3) & ~3) * 4 + (size_t)((rpw * bt + 3) & ~3) * 4 + (size_t)dw * kWave * vec * 4;
+  return (size_t)bt * nchv * 16 + (kFusedPool ? 2 : 1) * (size_t)((cap + 3) & ~3) * 4 + (size_t)((cap * bt + 3) & ~3) * 4 +
+         (size_t)dw * kWave * vec * 4;
+}
+// Slots a workgroup needs: its own share (tickets start after the two fixed neurons of every row wave), every neuron of
+// its group's pool, and one slot per row wave for the ticket that finds the pool empty.
+inline int fused_slot_cap(int spw, int rpw, int rw, bool pooled) {
+  if (!pooled) return rpw;
+  return (spw > 2 * rw ? spw : 2 * rw) + kFusedGroup * (rpw - spw) + rw;
 }
 
 enum FusedSlot { kSlotPending = 0, kSlotDead = 1, kSlotAnnounced = 2, kSlotLive = 3 };
@@ -61,12 +78,15 @@ struct FusedArgs {
   float* partial;        // [grid][nb][H] fp32
   float* y32;            // optional (nb, H) fp32: the workgroup adds its sums here with atomics instead of storing `partial`
   int32_t* counts;       // [grid] live neurons per workgroup
+  int32_t* pool;         // optional [groups][kPoolStride], all zero between calls: see the pool description at the kernel
   const u32x4* norm_w;   // optional (H,) RMS-norm weight applied to x while it is staged
   float norm_eps;
   int H, I, nb;
   int nch;               // 64-lane vector chunks per row: ceil(row_vecs / 64)
   int row_vecs;          // H / VEC
-  int rpw;               // neurons per workgroup
+  int rpw;               // neurons per workgroup (its own share and its part of the group's pool)
+  int spw;               // of those, the workgroup's own share; == rpw without a pool
+  int cap;               // slots per workgroup
   float t;               // threshold, already rounded through dtype
 #ifdef CATS_TIMING
   long long* tbuf;       // [gridDim][8] wall-clock stamps (100 MHz), development builds only
@@ -118,17 +138,22 @@ __device__ __forceinline__ void fused_dot(const u32x4 (&wv)[CB], const u32x4* xs
 template <int B, int KV, int RB>
 struct DownBatch {
   int rows[RB];       // neuron index, -1 = empty slot
+  int slots[RB];      // the slot the neuron was published in
   float zz[RB][B];
   int cnt;
   int unresolved;     // bit u: row u was taken while only announced, its z is still to be fetched
   u32x4 wv[RB][KV];
 };
 
-// Where the down waves read what the row waves publish: slot i is neuron row0 + i.
+// Where the down waves read what the row waves publish.  Slots are handed out in ticket order; the first slots are the
+// workgroup's own share in neuron order, those after it hold neurons taken from the group's pool.
 struct FusedSlots {
-  int* state;    // [n] FusedSlot; written and read with workgroup-scope atomics
-  float* z;      // [n][B]; ordered against state by LDS-only release / acquire fences
-  int row0, n;
+  int* state;    // [cap] FusedSlot; written and read with workgroup-scope atomics
+  float* z;      // [cap][B]; ordered against state by LDS-only release / acquire fences
+  int* row;      // pool build only: [cap] neuron of the slot, written before the slot leaves the pending state
+  int* nfinal;   // pool build only: number of slots in use; an upper bound (cap) until the last row wave has left
+  int cap;
+  int row0;      // neuron of slot 0 (slot i of the workgroup's own share is neuron row0 + i)
 };
 
 // Fill the batch with the next neurons that some batch row keeps, in neuron order, as far as the slots are decided.
@@ -137,8 +162,9 @@ struct FusedSlots {
 // Non-blocking: take what is there, possibly nothing.
 // The wave looks at 64 slots per pass -- lane i reads state and z of slot head + i, ballots find the decided prefix and
 // the kept slots in it -- so a pass costs one LDS round trip however many dead slots it steps over.
+// n: the caller's copy of the number of slots in use, refreshed here.
 template <int B, int KV, int RB>
-__device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const FusedSlots& sl, int& head, bool blocking) {
+__device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const FusedSlots& sl, int& head, int& n, bool blocking) {
   bt.cnt = 0;
   bt.unresolved = 0;
 #pragma unroll
@@ -148,11 +174,14 @@ __device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const Fu
     for (int b = 0; b < B; b++) bt.zz[u][b] = 0.f;
   }
   const int lane = threadIdx.x & (kWave - 1);
-  while (head < sl.n) {
+  for (;;) {
     const int idx = head + lane;
-    const bool in = idx < sl.n;  // never read past the slot array
+    const bool in = idx < sl.cap;  // never read past the slot array
     // past the end counts as pending: it ends the decided prefix
-    const int st_ = in ? __hip_atomic_load(&sl.state[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : kSlotPending;
+    int st_ = in ? __hip_atomic_load(&sl.state[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : kSlotPending;
+    if (kFusedPool) n = __builtin_amdgcn_readfirstlane(__hip_atomic_load(sl.nfinal, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
+    if (head >= n) return;
+    if (idx >= n) st_ = kSlotPending;  // slots past the last one in use may never have been written
     const uint64_t pend = __ballot(st_ == kSlotPending);
     uint64_t live = __ballot(st_ >= kSlotAnnounced);
     const uint64_t hasz = __ballot(st_ == kSlotLive);
@@ -167,13 +196,15 @@ __device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const Fu
     int zv[B];
 #pragma unroll
     for (int b = 0; b < B; b++) zv[b] = in ? __builtin_bit_cast(int, sl.z[idx * B + b]) : 0;
+    const int rowv = kFusedPool ? (in ? sl.row[idx] : -1) : sl.row0 + idx;
     if (ready < kWave) live &= (1ull << ready) - 1ull;
 #pragma unroll
     for (int u = 0; u < RB; u++) {
       if (live) {  // uniform
         const int bit = __builtin_ctzll(live);
         live &= live - 1ull;
-        bt.rows[u] = sl.row0 + head + bit;
+        bt.rows[u] = __builtin_amdgcn_readlane(rowv, bit);
+        bt.slots[u] = head + bit;
         if ((hasz >> bit) & 1ull) {
 #pragma unroll
           for (int b = 0; b < B; b++) bt.zz[u][b] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zv[b], bit));
@@ -198,7 +229,7 @@ __device__ __forceinline__ void fused_resolve(DownBatch<B, KV, RB>& bt, const Fu
   int myslot = -1;
 #pragma unroll
   for (int u = 0; u < RB; u++)
-    if (lane == u && ((bt.unresolved >> u) & 1)) myslot = bt.rows[u] - sl.row0;
+    if (lane == u && ((bt.unresolved >> u) & 1)) myslot = bt.slots[u];
   for (;;) {
     const int st_ = myslot >= 0 ? __hip_atomic_load(&sl.state[myslot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) : kSlotLive;
     if (__ballot(st_ != kSlotLive) == 0ull) break;
@@ -254,6 +285,9 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   constexpr int kXPre = 2;  // x vectors per thread fetched ahead of the first weight block
   extern __shared__ u32x4 s_fused[];
   __shared__ int s_ticket;
+  __shared__ int s_nfinal;     // slots in use; an upper bound while row waves are still taking tickets
+  __shared__ int s_exited;     // row waves that have left
+  __shared__ int s_exhausted;  // some row wave has found the group's pool empty
   __shared__ float s_scale[B];
 
   const int tid = threadIdx.x;
@@ -262,16 +296,32 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   const int nchp = (p.nch + CB - 1) / CB * CB;
   const int nchv = nchp * kWave;        // padded vectors per staged x row
   const int vlast = p.row_vecs - 1;
-  const int row0 = blockIdx.x * p.rpw;
-  const int n = min(p.rpw, p.I - row0);  // neurons of this workgroup (>= 1 by the launch shape)
+  // Neurons.  kFusedGroup consecutive workgroups form a group that owns kFusedGroup * rpw consecutive neurons.  Each
+  // workgroup has spw of them to itself; what is left at the end of the group's range is the group's pool, handed out
+  // one neuron at a time (a ticket counter in memory) to whichever row wave of the group asks first once its
+  // workgroup's own share is taken.  Workgroups that got few live neurons, or a fast XCD, end up with more of the pool.
+  // Without a pool (spw == rpw) this is one contiguous share per workgroup.
+  const bool pooled = kFusedPool && p.pool != nullptr;
+  const int grp = blockIdx.x / kFusedGroup, gi = blockIdx.x - grp * kFusedGroup;
+  const int g0 = grp * kFusedGroup * p.rpw;
+  const int ng = min(p.I - g0, kFusedGroup * p.rpw);             // neurons of the group (>= 1 by the launch shape)
+  const int gsz = min(kFusedGroup, (int)gridDim.x - grp * kFusedGroup);  // workgroups of the group
+  const int row0 = g0 + gi * p.spw;
+  const int n = max(0, min(p.spw, ng - gi * p.spw));             // neurons of this workgroup's own share
+  const int pool0 = g0 + gsz * p.spw;
+  const int psize = max(0, ng - gsz * p.spw);                    // neurons in the pool
+  int32_t* const pool_ctr = pooled ? p.pool + (size_t)grp * kPoolStride : p.counts;  // only touched when pooled
 
   u32x4* xs = s_fused;                                       // [B][nchv]
+  const int cap4 = (p.cap + 3) & ~3;
   FusedSlots sl;
-  sl.state = (int*)(s_fused + B * nchv);          // [rpw]
-  sl.z = (float*)(sl.state + ((p.rpw + 3) & ~3));  // [rpw][B]
+  sl.state = (int*)(s_fused + B * nchv);  // [cap]
+  sl.row = sl.state + cap4;               // [cap], pool build only
+  sl.z = (float*)(sl.state + (kFusedPool ? 2 : 1) * cap4);  // [cap][B]
+  sl.nfinal = &s_nfinal;
+  sl.cap = p.cap;
   sl.row0 = row0;
-  sl.n = n;
-  float* tr_all = sl.z + ((p.rpw * B + 3) & ~3);   // [DW][64 * VEC]: where a down wave regroups its sums by column (y32 mode)
+  float* tr_all = sl.z + ((p.cap * B + 3) & ~3);   // [DW][64 * VEC]: where a down wave regroups its sums by column (y32 mode)
 
   CATS_FSTAMP(tid == 0, 0);
   const bool is_row_wave = wave >= DW;
@@ -305,11 +355,19 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       if (b < p.nb && v < p.row_vecs) val = p.x[(size_t)b * p.row_vecs + v];
       xs[i] = val;
     }
-    // given activations: the down waves decide every slot (announced or dead) while they stage the activations
+    // given activations: the down waves decide every slot (announced or dead) while they stage the activations.
+    // Tickets start at 2 * RW: the slots between a short share and that point are never taken.
     if (gate)
-      for (int i = tid; i < p.rpw; i += kFusedThreads) sl.state[i] = kSlotPending;
+      for (int i = tid; i < p.cap; i += kFusedThreads) sl.state[i] = (i >= n && i < 2 * RW) ? kSlotDead : kSlotPending;
+    if (kFusedPool)
+      for (int i = tid; i < n; i += kFusedThreads) sl.row[i] = row0 + i;
     // gate mode: the first two neurons of every row wave are fixed, the rest go by ticket; given activations: all by ticket
-    if (tid == 0) s_ticket = gate ? 2 * RW : 0;
+    if (tid == 0) {
+      s_ticket = gate ? 2 * RW : 0;
+      s_nfinal = (gate && pooled) ? p.cap : n;
+      s_exited = 0;
+      s_exhausted = 0;
+    }
     __syncthreads();
     if (p.norm_w) {
       // RMS norm of each batch row, in place in LDS: one wave adds a row's squares (fixed order), everyone rescales.
@@ -422,8 +480,11 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   if (is_row_wave) {
     // ---- row waves: gate -> decision -> up -> publish ------------------------------------------------------------
     // A wave holds its current neuron, the next one (whose first gate block it prefetches) and the ticket after that.
-    int cur = neuron_of(rw);
-    int nxt = neuron_of(rw + RW);
+    // A ticket past the workgroup's own share is exchanged for a neuron of the group's pool; the request to the pool's
+    // counter in memory goes out with the ticket and has a whole neuron's time to come back.
+    int cur = neuron_of(rw), curslot = rw;
+    int nxt = neuron_of(rw + RW), nxtslot = rw + RW;
+    bool last_ticket = false;  // this wave has taken its last ticket
     u32x4 wc[CB];
     stage([&] {
       const u32x4* src = cur >= 0 ? p.wg + (size_t)cur * p.row_vecs : p.x;
@@ -431,8 +492,18 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
     });
     const int nblk = nchp / CB;
     while (cur >= 0) {
-      int pend = 0;
-      if (lane == 0) pend = __hip_atomic_fetch_add(&s_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      int pend = -1, pticket = 0;
+      bool ask_pool = false;
+      if (!last_ticket) {
+        int gone = 0;
+        if (lane == 0) {
+          pend = __hip_atomic_fetch_add(&s_ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          gone = __hip_atomic_load(&s_exhausted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+        pend = __builtin_amdgcn_readfirstlane(pend);
+        ask_pool = pooled && pend >= n && __builtin_amdgcn_readfirstlane(gone) == 0;
+        if (ask_pool && lane == 0) pticket = __hip_atomic_fetch_add(pool_ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
       const int row = cur;
       float a[B];
       bool act[B];
@@ -467,7 +538,7 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
 #endif
       if (any) {  // wave-uniform
         // the down waves may send for this neuron's W_down^T row now: it travels while the W_up row does
-        if (lane == 0) __hip_atomic_store(&sl.state[row - row0], kSlotAnnounced, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (lane == 0) __hip_atomic_store(&sl.state[curslot], kSlotAnnounced, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         float u[B];
 #pragma unroll
         for (int b = 0; b < B; b++) u[b] = 0.f;
@@ -489,7 +560,7 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
           for (int b = 0; b < B; b++)
             if (b < p.nb) p.flag_out[(size_t)b * p.I + row] = act[b] ? 1 : 0;
         }
-        const int slot = row - row0;
+        const int slot = curslot;
 #pragma unroll
         for (int b = 0; b < B; b++) sl.z[slot * B + b] = z[b];
         // release side (LDS only, so the gate rows in flight are not waited for): z is in LDS before the state says so
@@ -497,11 +568,52 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
         __hip_atomic_store(&sl.state[slot], any ? kSlotLive : kSlotDead, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
       cur = nxt;
-      nxt = neuron_of(__builtin_amdgcn_readfirstlane(pend));
+      curslot = nxtslot;
+      // what the ticket taken at the top of this round is worth
+      nxt = -1;
+      nxtslot = pend;
+      if (pend >= 0) {  // wave-uniform
+        if (pend < n) {
+          nxt = row0 + pend;
+        } else {
+          last_ticket = true;  // unless the pool gives a neuron
+          if (ask_pool) {
+            const int g = __builtin_amdgcn_readfirstlane(pticket);
+            if (g < psize) {
+              nxt = pool0 + g;
+              last_ticket = false;
+            }
+          }
+          if (pooled && lane == 0) {
+            // the slot is taken either way: it gets the pool's neuron (written before any state that lets a down wave
+            // look at it: same wave, LDS keeps a wave's accesses in order), or it is dead
+            if (nxt >= 0) {
+              sl.row[pend] = nxt;
+            } else {
+              __hip_atomic_store(&sl.state[pend], kSlotDead, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+              __hip_atomic_store(&s_exhausted, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+          }
+        }
+      }
     }
 #ifdef CATS_TIMING
     if (p.tbuf && lane == 0) atomicMax((unsigned long long*)&p.tbuf[(size_t)blockIdx.x * 8 + 2], (unsigned long long)wall_clock64());
 #endif
+    if (pooled && lane == 0) {
+      // The last row wave to leave knows how many slots were handed out: no ticket is taken after this point.  It also
+      // reports the workgroup to its group; the last workgroup of the group to do so puts both counters back to zero
+      // for the next call (every ticket of this call has been taken by then).
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+      if (__hip_atomic_fetch_add(&s_exited, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) == RW - 1) {
+        const int used = __hip_atomic_load(&s_ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        __hip_atomic_store(&s_nfinal, used, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (__hip_atomic_fetch_add(pool_ctr + 16, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gsz - 1) {
+          __hip_atomic_store(pool_ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(pool_ctr + 16, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+    }
     return;
   }
 
@@ -536,13 +648,14 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       for (int e = 0; e < VEC; e++) acc[b][k][e] = 0.f;
 
   int head = 0, nlive = 0;
+  int nfin = kFusedPool ? p.cap : n;  // slots in use, as far as this wave knows (the pool build refreshes it in fused_collect)
   DownBatch<B, KV, RB> ba, bb;
-  fused_collect<B, KV, RB>(ba, sl, head, true);
+  fused_collect<B, KV, RB>(ba, sl, head, nfin, true);
   fused_down_issue<B, KV, RB>(ba, p.wd, p.row_vecs, p.x, vidx);
   for (;;) {
-    if (ba.cnt == 0 && head >= n) break;
-    fused_collect<B, KV, RB>(bb, sl, head, ba.cnt == 0);
-    if (bb.cnt == 0 && head >= n) {
+    if (ba.cnt == 0 && head >= nfin) break;
+    fused_collect<B, KV, RB>(bb, sl, head, nfin, ba.cnt == 0);
+    if (bb.cnt == 0 && head >= nfin) {
       // nothing left to send for: finish the batch in flight and leave no load behind (whatever is still outstanding
       // when the sums are written out has to be waited for first)
       fused_resolve<B, KV, RB>(ba, sl);
@@ -555,8 +668,8 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
     fused_resolve<B, KV, RB>(ba, sl);
     fused_down_consume<DT, B, KV, RB>(ba, acc);
     nlive += ba.cnt;
-    fused_collect<B, KV, RB>(ba, sl, head, bb.cnt == 0);
-    if (ba.cnt == 0 && head >= n) {
+    fused_collect<B, KV, RB>(ba, sl, head, nfin, bb.cnt == 0);
+    if (ba.cnt == 0 && head >= nfin) {
       fused_resolve<B, KV, RB>(bb, sl);
       fused_down_consume<DT, B, KV, RB>(bb, acc);
       nlive += bb.cnt;

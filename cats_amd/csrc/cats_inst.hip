@@ -47,8 +47,7 @@ hipError_t launch_rows_one(const RowsArgs& a, hipStream_t stream) {
   size_t lds = XLDS ? (size_t)B * ((a.nch + kCB - 1) / kCB * kCB) * kWave * sizeof(u32x4) : 0;
   if ((size_t)a.lds_floor > lds) lds = (size_t)a.lds_floor;
   if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(WAVES * kWave), lds, stream, a);
-  return hipGetLastError();
+  return launch_kernel(kern, dim3(grid), dim3(WAVES * kWave), lds, stream, a);
 }
 
 // Matrix-core gate + up pass: one persistent workgroup per CU.
@@ -71,8 +70,7 @@ struct MmaLaunch16 {
     const size_t lds = rows_mma_lds_bytes(a.K);
     if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
     const int ntiles = (a.N + kMmaTileRows - 1) / kMmaTileRows;
-    hipLaunchKernelGGL(kern, dim3(ntiles < cus ? ntiles : cus), dim3(kMmaThreads), lds, stream, a);
-    return hipGetLastError();
+    return launch_kernel(kern, dim3(ntiles < cus ? ntiles : cus), dim3(kMmaThreads), lds, stream, a);
   }
 };
 template <> struct MmaLaunch<F16> : MmaLaunch16<F16> {};
@@ -81,8 +79,7 @@ template <> struct MmaLaunch<BF16> : MmaLaunch16<BF16> {};
 template <class DT, int B>
 hipError_t launch_rows_b(int mode, const RowsArgs& a, hipStream_t stream) {
   // measured on Llama-7B shapes: at 2 batch rows the wave-per-row kernel is still the faster one (28.4 vs 29.4 us)
-  // The plain gate pass goes the same way (unless the caller wants the compact index list, which is a batch-1
-  // feature), so a gate call and a fused call produce the same activations bit for bit.
+  // The plain gate pass goes the same way, so a gate call and a fused call produce the same activations bit for bit.
   if ((mode == kGateUp || mode == kGate) && B >= 4 && a.mma && MmaLaunch<DT>::supported(a))
     return MmaLaunch<DT>::run(a, mode == kGateUp, stream);
   const size_t lds = (size_t)B * ((a.nch + kCB - 1) / kCB * kCB) * kWave * sizeof(u32x4);
@@ -121,17 +118,15 @@ hipError_t launch_down_one(const DownArgs& a, int block, hipStream_t stream) {
   const size_t lds_fold = (size_t)nwaves * (B < 4 ? B : 4) * kWave * DT::VEC * sizeof(float);  // up to four batch rows per pass
   const size_t lds = (lds_stream > lds_fold ? lds_stream : lds_fold) + 64;
   if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, dim3(a.nslab * a.ngroup), dim3(block), lds, stream, a);
-  return hipGetLastError();
+  return launch_kernel(kern, dim3(a.nslab * a.ngroup), dim3(block), lds, stream, a);
 }
 
 template <class DT, int B, bool FULL, int KV, int DW>
 hipError_t launch_fused_one(int grid, const FusedArgs& a, hipStream_t stream) {
   auto kern = mlp_fused_kernel<DT, B, FULL, KV, DW>;
-  const size_t lds = fused_lds_bytes(B, a.nch, a.rpw, DT::VEC, DW);
+  const size_t lds = fused_lds_bytes(B, a.nch, a.cap, DT::VEC, DW);
   if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kFusedThreads), lds, stream, a);
-  return hipGetLastError();
+  return launch_kernel(kern, dim3(grid), dim3(kFusedThreads), lds, stream, a);
 }
 
 template <class DT, int B>
@@ -159,8 +154,7 @@ hipError_t launch_fused<CATS_DT>(int bt, int grid, int stage, const FusedArgs& a
   }
   if (stage != 1) {
     const int rgrid = (r.BH + kReduceCols - 1) / kReduceCols;  // BH == 0: only the count is wanted
-    hipLaunchKernelGGL(reduce_partials_kernel<CATS_DT>, dim3(rgrid > 0 ? rgrid : 1), dim3(256), 0, stream, r);
-    return hipGetLastError();
+    return launch_kernel(reduce_partials_kernel<CATS_DT>, dim3(rgrid > 0 ? rgrid : 1), dim3(256), 0, stream, r);
   }
   return hipSuccess;
 }

@@ -18,6 +18,15 @@ struct Tuning {
 // Compute units of the current device (256 if the runtime will not say), remembered per device.
 int current_device_cus();
 
+// Launch a kernel and return the status of this launch alone.  (hipGetLastError() after a <<<>>> launch would also
+// return, and clear, an error that some earlier call of the caller left behind.)  Every argument must already have
+// the kernel's parameter type.
+template <class K, class... A>
+inline hipError_t launch_kernel(K kern, dim3 grid, dim3 block, size_t lds, hipStream_t stream, A... a) {
+  void* params[] = {(void*)&a...};
+  return hipLaunchKernel((const void*)kern, grid, block, params, lds, stream);
+}
+
 // Returns hipSuccess or the launch error.  `mode` is a RowsMode; bt (1, 2, 4 or 8) the compile-time batch.
 template <class DT>
 hipError_t launch_rows(int mode, int bt, const RowsArgs& a, hipStream_t stream);

@@ -86,7 +86,9 @@ class CatsMLP(nn.Module):
         self.visit_counts = 0
         self.count = 0
         self.t = 0
-        self.decode_fetched: Optional[torch.Tensor] = None  # neurons fetched by the kernel path while is_stats (device int64)
+        # kernel path while is_stats: [neurons fetched, calls] as one device int64 pair.  Both are added to on the device,
+        # so a HIP-graph replay of the decode step counts the call as well as the neurons.
+        self.decode_fetched: Optional[torch.Tensor] = None
         self.histogram_bins = histogram_bins()
         self.pre_act_hist_counts = torch.zeros(NUM_BINS - 1)
         self.post_act_hist_counts = torch.zeros(NUM_BINS - 1)
@@ -105,9 +107,12 @@ class CatsMLP(nn.Module):
     def decode_union_sparsity(self) -> Optional[float]:
         """1 - (neurons fetched per call) / I over the kernel-path calls made while is_stats; None if there were none.
         This is what the reference's microbenchmark reports as sparsity (flash_gemv/bench/profile_llama7B.py:56,72)."""
-        if self.decode_fetched is None or self.visit_counts == 0:
+        if self.decode_fetched is None:
             return None
-        return 1.0 - float(self.decode_fetched.item()) / (self.visit_counts * self.intermediate_size)
+        fetched, calls = (int(v) for v in self.decode_fetched.tolist())
+        if calls == 0:
+            return None
+        return 1.0 - fetched / (calls * self.intermediate_size)
 
     def collect_stats(self, pre_activation, post_activation):
         start_time = time.time()
@@ -167,9 +172,9 @@ class CatsMLP(nn.Module):
                     # the running total stays on the device, so nothing here waits for the GPU
                     y, _, fetched = flash_gemv.cats_mlp_stats(x, self.gate_proj.weight, self.up_proj.weight, self.wdown_t, t)
                     if self.decode_fetched is None or self.decode_fetched.device != fetched.device:
-                        self.decode_fetched = torch.zeros((), dtype=torch.int64, device=fetched.device)
-                    self.decode_fetched += fetched
-                    self.visit_counts += 1
+                        self.decode_fetched = torch.zeros(2, dtype=torch.int64, device=fetched.device)
+                    self.decode_fetched[0] += fetched.reshape(())
+                    self.decode_fetched[1] += 1
                     return y
                 return flash_gemv.cats_mlp(x, self.gate_proj.weight, self.up_proj.weight, self.wdown_t, t)
             return self._dense_masked(x)

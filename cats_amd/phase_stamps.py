@@ -1,7 +1,7 @@
 """Where the time of the single-pass MLP kernel goes, workgroup by workgroup.
 
 ``python -m cats_amd.phase_stamps [--batch 1] [--sparsity 0.5] [--calls 24]`` loads the stamped twin of the kernel
-library (``cats_amd/lib/libcats_gemv_timing.so``, built by ``python -m cats_amd.build`` with ``-DCATS_TIMING``), runs
+library (``cats_amd/lib/libcats_gemv_timing.so``, built by ``python -m cats_amd.build --timing`` with ``-DCATS_TIMING``), runs
 ``cats_mlp`` on the Llama-2-7B layer shape over rotating weight sets and prints, over all workgroups of all calls,
 when each phase boundary was reached (microseconds after the first workgroup of the call started; the stamp is the
 100 MHz ``wall_clock64`` counter, so one tick is 10 ns):

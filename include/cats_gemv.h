@@ -3,7 +3,10 @@
  *
  * Every entry point takes plain device pointers, sizes and a HIP stream and returns a
  * cats_status_t.  Nothing here allocates, frees or synchronises (cats_read_count is the one
- * documented exception: it has to hand a device counter back to the host).  All launches go
+ * documented exception: it has to hand a device counter back to the host, and its first call
+ * allocates one pinned host word for that).  A launch failure is reported as CATS_ERR_LAUNCH
+ * from the status of that launch alone; errors left behind by the caller's earlier HIP calls are
+ * neither returned nor cleared.  All launches go
  * to the stream that is passed in.  The entry points are what a `TORCH_LIBRARY(flash_gemv, m)`
  * shim, a ctypes loader or any other FFI binds; each one names the reference interface it
  * stands in for (paths relative to the CATS tree).
@@ -65,7 +68,8 @@ const char* cats_status_string(int status);
  * gate activations of the list-building call.  Replaces the per-call cudaMalloc/cudaFree pairs of the reference
  * (fuse_gemv_cmp_cuda.cu:2351-2354,2402-2403).  The caller allocates cats_workspace_bytes() once (256-byte
  * aligned), runs cats_workspace_init() once (it zero-fills with a kernel), and then passes the same buffer to
- * every call; no call relies on what an earlier call left in it.  The size and the carving depend on (H, I)
+ * every call; no call relies on what an earlier call left in it (the counter words at its head are all zero
+ * between calls: a call that uses them puts them back).  The size and the carving depend on (H, I)
  * only (B is checked; every region holds the 8 rows of one pass over the weights, and a call with 9..16 rows
  * reuses them pass by pass), so one workspace serves every batch size of one layer shape; for another (H, I)
  * use another workspace or initialise again.  One workspace serves one stream at a time. */
@@ -87,7 +91,8 @@ int cats_gate_flag(const void* x, const void* wgate, void* a_out, uint8_t* flag_
 int cats_gate_compact(const void* x, const void* wgate, void* vals_out, int64_t* idx_out, int32_t* count_out,
                       int H, int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream);
 
-/* Blocking helper for the call above: waits for the stream and returns *count_dev (or -1 on error). */
+/* Blocking helper for the call above: copies *count_dev to pinned host memory behind the work already on the
+ * stream, waits for the stream once and returns the value (or -1 on error). */
 int cats_read_count(const int32_t* count_dev, void* stream);
 
 /* Sparse up projection over a flag array.  out[b,j] = flag[b,j] ? a[b,j] * (x[b,:] . wup[j,:]) : 0.
