@@ -7,10 +7,12 @@ the configuration the headline metric is quoted on.  Inputs are resident in HBM 
 Steps rotate over several independent weight sets whose total size exceeds the 256 MB memory-side cache,
 so every step streams its weights from HBM.
 
-Prints ONE JSON line: per-layer latency (value, us), achieved HBM bandwidth on touched bytes, the same for
-sparsities 0/30/50/70/90 %, the dense fp16 GEMV MLP (stock PyTorch-ROCm F.linear) on the same GPU, a
-`roofline` object for the dominant kernel and a `cpu_baseline` object (the dense-masked PyTorch CATS MLP on
-this box's host cores).  `--decode` adds the 32-layer decode loop (tokens/s, CATS vs dense).
+Prints ONE JSON line: per-layer latency (value, us: plain stream launches of the fp16-output call; the HIP-graph
+replay and the one-launch fp32-accumulate contract beside it), achieved HBM bandwidth on touched bytes, the same
+for sparsities 0/30/50/70/90 %, the dense fp16 GEMV MLP (stock PyTorch-ROCm F.linear) on the same GPU, the read-stream
+bandwidth the GPU reaches (`stream_ceiling`), a `roofline` object for the dominant kernel and a `cpu_baseline` object
+(the dense-masked PyTorch CATS MLP on this box's host cores).  `--decode` adds the 32-layer decode loop (tokens/s,
+CATS vs dense).
 """
 from __future__ import annotations
 
@@ -41,13 +43,14 @@ def touched_bytes(sz, B, k):
 
 
 def stage_bytes(sz, B, k, grid=256):
-    """Algorithmic bytes per launch of the two kernels of the single-pass path: (streaming kernel, reduction).
-    Streaming: all of W_gate, k rows each of W_up and W_down^T, x, and the fp32 partial sums it leaves per workgroup;
-    reduction: those partial sums and y."""
+    """Bytes per launch of the two kernels of the single-pass path: (streaming kernel, reduction, partial sums).
+    Streaming: the algorithmic bytes of the whole call (touched_bytes: the streaming kernel is the one that moves them);
+    the fp32 partial sums it leaves per workgroup are this design's own overhead and are returned separately, not
+    counted as algorithmic.  Reduction: those partial sums and y."""
     partials = grid * B * H * 4
-    stream = sz * H * I + 2 * sz * H * k + sz * B * H + partials
+    stream = touched_bytes(sz, B, k)
     reduce = partials + sz * B * H
-    return stream, reduce
+    return stream, reduce, partials
 
 
 def csrc_hash():
@@ -149,9 +152,11 @@ def main():
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     p = lambda t: ctypes.c_void_p(t.data_ptr())
 
-    def mlp_args(st, t, cnt=None):
-        return (p(x), p(st["wg"]), p(st["wu"]), p(st["wdt"]), p(y), None, None, cnt, B, H, I, capi.F16, ctypes.c_float(t),
-                p(ws.buf), ws.nbytes, stream)
+    y32 = torch.zeros(B, H, dtype=torch.float32, device=dev)
+
+    def mlp_args(st, t, cnt=None, f32=False):
+        return (p(x), p(st["wg"]), p(st["wu"]), p(st["wdt"]), None if f32 else p(y), p(y32) if f32 else None, None, cnt, B, H, I,
+                capi.F16, ctypes.c_float(t), p(ws.buf), ws.nbytes, stream)
 
     def active_count(t):
         ks = []
@@ -173,13 +178,19 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e3 / steps  # us per step
 
-    def time_cats(t, steps, warmup, stage=0):
-        """stage 0: the whole call; 1 / 2: one of its two launches alone, back to back (cats_mlp_stage)."""
-        prepared = [mlp_args(st, t) for st in sets]
+    def time_cats(t, steps, warmup, stage=0, f32=False, zero_fill=False):
+        """stage 0: the whole call; 1 / 2: one of its two launches alone, back to back (cats_mlp_stage).
+        f32: the fp32-accumulate contract (one launch, atomics into the caller's buffer); zero_fill: with the fill
+        kernel that contract asks the caller for in front of every call."""
+        prepared = [mlp_args(st, t, f32=f32) for st in sets]
         n = len(prepared)
         if stage:
             stage_args = [(stage,) + a[:5] + a[8:] for a in prepared]  # no y_f32 / flag_out / count_out
             fn = lambda i: L.cats_mlp_stage(*stage_args[i % n])
+        elif zero_fill:
+            def fn(i):
+                y32.zero_()
+                return L.cats_mlp(*prepared[i % n])
         else:
             fn = lambda i: L.cats_mlp(*prepared[i % n])
         capi.check(fn(0), "cats_mlp (first timed-configuration call)")
@@ -256,13 +267,17 @@ def main():
     us_k2 = time_cats(t50, kernel_steps, kernel_warmup, stage=2)
     rep_stats = per_rep_stats(t50, min(400, max(50, args.steps)))
     us_dense = time_dense(args.steps, args.warmup)
-    us = us_eager if us_graph is None else min(us_eager, us_graph)
-    launch = "stream" if (us_graph is None or us_eager <= us_graph) else "hipgraph"
-    steps_timed = args.steps if launch == "stream" else graph_steps
+    us_f32 = time_cats(t50, args.steps, args.warmup, f32=True)
+    us_f32_zero = time_cats(t50, args.steps, args.warmup, f32=True, zero_fill=True)
+    # value is the plain stream-launch time of the call the decode path makes (fp16 y, two launches, bitwise
+    # reproducible); the graph replay and the one-launch fp32-accumulate contract are reported beside it
+    us, launch, steps_timed = us_eager, "stream", args.steps
     tb = touched_bytes(sz, B, k50)
+    ceiling = stream_ceiling(torch, capi)
     single_pass = args.path != 1
+    partial_bytes = 0
     if single_pass:
-        b_k1, b_k2 = stage_bytes(sz, B, k50)
+        b_k1, b_k2, partial_bytes = stage_bytes(sz, B, k50)
         k1_name = "cats::mlp_fused_kernel<F16,B=1> (gate GEMV + SiLU + threshold + sparse up + sparse down into per-workgroup partial sums)"
         k2_name = "cats::reduce_partials_kernel<F16> (sum of the 256 partial sums, rounding, y)"
     else:
@@ -278,12 +293,12 @@ def main():
         for s in SPARSITIES:
             k = active_count(thr[s])
             u = time_cats(thr[s], ssteps, swarm)
-            if not args.no_graph:
-                u = min(u, time_cats_graph(thr[s], ssteps, swarm)[0])
+            u32 = time_cats(thr[s], ssteps, swarm, f32=True)
             b = touched_bytes(sz, B, k)
             sweep.append(dict(target_sparsity=s, sparsity=round(1 - k / I, 4), us=round(u, 2), touched_MB=round(b / 1e6, 1),
                               GBps=round(b / u * 1e-3, 1), hbm_frac=round(b / u * 1e-3 / HBM_PEAK_GBPS, 4),
-                              speedup_vs_dense=round(us_dense / u, 3)))
+                              speedup_vs_dense=round(us_dense / u, 3), us_f32_accumulate=round(u32, 2),
+                              hbm_frac_f32_accumulate=round(b / u32 * 1e-3 / HBM_PEAK_GBPS, 4)))
 
     out = {
         "metric": "CATS-MLP us/layer + achieved HBM GB/s (touched bytes); batch-1 decode tok/s",
@@ -307,6 +322,18 @@ def main():
         "hbm_frac_touched": round(tb / us * 1e-3 / HBM_PEAK_GBPS, 4),
         "us_stream_launch": round(us_eager, 3),
         "us_hipgraph": None if us_graph is None else round(us_graph, 3),
+        "hipgraph_steps": graph_steps,
+        "f32_accumulate": {
+            "what": "cats_mlp with y_f32 (the contract of the reference's fuse_gemv_gemv_gemv / flag_gemv_gemv_atomic: the caller "
+                    "zeroes an fp32 (B, H) buffer, the call adds into it): one launch, fp32 atomics, no reduction launch; summation "
+                    "order and so the last bits vary from run to run",
+            "us": round(us_f32, 3),
+            "hbm_frac_touched": round(tb / us_f32 * 1e-3 / HBM_PEAK_GBPS, 4),
+            "us_with_zero_fill": round(us_f32_zero, 3),
+            "hbm_frac_touched_with_zero_fill": round(tb / us_f32_zero * 1e-3 / HBM_PEAK_GBPS, 4),
+        },
+        "stream_ceiling": ceiling,
+        "frac_of_stream_ceiling": round(tb / us * 1e-3 / ceiling["GBps"], 4),
         "dense_fp16_us": round(us_dense, 3),
         "dense_GBps": round(3 * sz * H * I / us_dense * 1e-3, 1),
         "speedup_vs_dense": round(us_dense / us, 3),
@@ -321,7 +348,12 @@ def main():
             "traffic": traffic,
             "traffic_source": traffic_note,
             "bytes_per_launch": int(b_k1),
+            "design_overhead_bytes": int(partial_bytes),
+            "bytes_note": "bytes_per_launch are the algorithmic bytes of the call (weights touched, x, y, a, index list, count); "
+                          "design_overhead_bytes are the per-workgroup fp32 partial sums this design writes and reads on top, "
+                          "not counted in achieved / frac",
             "us_per_launch": round(us_k1, 3),
+            "frac_of_stream_ceiling": round(b_k1 / us_k1 * 1e-3 / ceiling["GBps"], 4),
             "second_kernel": {"kernel": k2_name, "bytes_per_launch": int(b_k2), "us_per_launch": round(us_k2, 3),
                               "achieved": round(b_k2 / us_k2 * 1e-3, 1), "frac": round(b_k2 / us_k2 * 1e-3 / HBM_PEAK_GBPS, 4)},
             "kernel_launches_timed": kernel_steps,
@@ -358,6 +390,29 @@ def main():
     print(json.dumps(out))
 
 
+def stream_ceiling(torch, capi, gib=1, reps=40):
+    """Read-stream bandwidth this GPU reaches: cats_probe_read (read-only, the same 128-bit streaming loads as the weight
+    rows) over a 1 GiB buffer, four times the 256 MB memory-side cache, timed with events on the launch stream."""
+    buf = torch.empty(gib << 30, dtype=torch.uint8, device="cuda")
+    buf.fill_(1)
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    for _ in range(5):
+        capi.probe_read(buf, sink)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        capi.probe_read(buf, sink)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / reps
+    nbytes = buf.numel()
+    del buf
+    torch.cuda.empty_cache()
+    return {"GBps": round(nbytes / us * 1e-3, 1), "frac_of_peak": round(nbytes / us * 1e-3 / HBM_PEAK_GBPS, 4), "bytes": nbytes,
+            "us_per_pass": round(us, 2), "kernel": "read_probe_kernel (cats_probe_read): read-only, nothing written"}
+
+
 def other_configs(torch, F, capi, L, steps, warmup, which):
     """The remaining single-layer configurations: Mistral-7B shape in bf16 with heavy-tailed gate rows (50 / 70 %), and
     the Llama fp16 layer at batch 2 / 4 / 8 with pairwise-correlated rows (per-row masks, union gathering), and the
@@ -387,6 +442,7 @@ def other_configs(torch, F, capi, L, steps, warmup, which):
         act = F.silu(X @ sets[0]["wg"].float().t()).abs().flatten().cpu()
         ws = capi.Workspace(B, Hh, Ii)
         y = torch.empty(B, Hh, dtype=dtype, device=dev)
+        y32 = torch.zeros(B, Hh, dtype=torch.float32, device=dev)
         count = torch.zeros(1, dtype=torch.int32, device=dev)
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         p = lambda t: ctypes.c_void_p(t.data_ptr())
@@ -415,10 +471,14 @@ def other_configs(torch, F, capi, L, steps, warmup, which):
             prepared = [(p(x), p(st["wg"]), p(st["wu"]), p(st["wdt"]), p(y), None, None, None, B, Hh, Ii, code, ctypes.c_float(t), p(ws.buf), ws.nbytes, stream)
                         for st in sets]
             us = timed(lambda i: L.cats_mlp(*prepared[i % nsets]))
+            # the fp32-accumulate contract (adds into the caller's fp32 buffer; one launch at 1..2 rows)
+            prepared32 = [a[:4] + (None, p(y32)) + a[6:] for a in prepared]
+            us32 = timed(lambda i: L.cats_mlp(*prepared32[i % nsets]))
             tb = sz * Hh * Ii + 2 * sz * Hh * k + sz * B * (2 * Hh + Ii) + 4 * k + 4
             res.append(dict(config=name, batch=B, row_sparsity_target=s, union_sparsity=round(1 - k / Ii, 4), us=round(us, 2),
                             touched_MB=round(tb / 1e6, 1), GBps=round(tb / us * 1e-3, 1), hbm_frac=round(tb / us * 1e-3 / HBM_PEAK_GBPS, 4),
-                            dense_us=round(us_dense, 2), speedup_vs_dense=round(us_dense / us, 3)))
+                            dense_us=round(us_dense, 2), speedup_vs_dense=round(us_dense / us, 3), us_f32_accumulate=round(us32, 2),
+                            hbm_frac_f32_accumulate=round(tb / us32 * 1e-3 / HBM_PEAK_GBPS, 4)))
         del sets
         torch.cuda.empty_cache()
 
@@ -465,6 +525,7 @@ def entry_points(torch, F, capi, steps, warmup, only=()):
     vals = torch.empty(I, dtype=torch.float16, device=dev)
     idx = torch.empty(I, dtype=torch.int64, device=dev)
     cnt = torch.zeros(1, dtype=torch.int32, device=dev)
+    out32 = torch.zeros(1, H, dtype=torch.float32, device=dev)
     L = capi.lib()
     import flash_gemv as fg
 
@@ -501,10 +562,55 @@ def entry_points(torch, F, capi, steps, warmup, only=()):
          full + 2 * act_rows, lambda st: fg.flag_gemv_gemv_dejavu(x, st["wg_t"], st["wu"], st["wdt"], t)),
         ("cats_up_down", "gemv_gemv_triton (gate activations given)", 2 * act_rows, lambda st: capi.up_down(x, st["a"], st["wu"], st["wdt"], t, ws)),
         ("cats_gate_up", "fuse_gemv_flag_gemv", full + act_rows, lambda st: capi.gate_up(x, st["wg"], st["wu"], t)),
-        ("cats_mlp", "flag_gemv_gemv_atomic, fuse_gemv_flag_gemv_gemv", full + 2 * act_rows, lambda st: capi.mlp(x, st["wg"], st["wu"], st["wdt"], t, ws)),
+        ("cats_mlp", "the whole MLP into an fp16 y (no single reference op; what flash_gemv.cats_mlp and CatsMLP sp_method 3 call)",
+         full + 2 * act_rows, lambda st: capi.mlp(x, st["wg"], st["wu"], st["wdt"], t, ws)),
+        ("cats_mlp (y_f32)", "the C call behind flag_gemv_gemv_atomic / fuse_gemv_gemv_gemv / fuse_gemv_flag_gemv_gemv: adds into an fp32 y",
+         full + 2 * act_rows, lambda st: capi.mlp(x, st["wg"], st["wu"], st["wdt"], t, ws, y_f32=out32)),
         ("cats_mlp_norm_residual", "norm -> mlp -> residual of the decoder layer", full + 2 * act_rows,
          lambda st: capi.mlp_norm_residual(x, nw, 1e-5, st["wg"], st["wu"], st["wdt"], t, ws)),
         ("cats_mlp_rowmajor_down", "flag_gemv_gemv, flag_gemv_gemv_inner*", 2 * full + act_rows, lambda st: capi.mlp_rowmajor_down(x, st["wg"], st["wu"], st["wd"], t, ws)),
+    ]
+    # the registered torch ops and the Python composites, called as a user of the reference's package calls them
+    x3 = x.reshape(1, 1, H)
+    act_fn = torch.nn.SiLU()
+    flag1 = torch.zeros(1, I, dtype=torch.bool, device=dev)
+
+    def zeroed(op):
+        def call(st):
+            out32.zero_()   # the contract of these ops: the caller zeroes the fp32 output
+            return op(st)
+        return call
+
+    def module_call(method):
+        from cats_amd.mlp import CatsMLP
+
+        mods = []
+        for st in sets:
+            m = CatsMLP(H, I, dead_threshold=t, dtype=torch.float16, device="meta")
+            m.gate_proj.weight = torch.nn.Parameter(st["wg"], requires_grad=False)
+            m.up_proj.weight = torch.nn.Parameter(st["wu"], requires_grad=False)
+            m.down_proj.weight = torch.nn.Parameter(st["wd"], requires_grad=False)
+            m.is_profile, m.sp_method, m.wdown_t = True, method, st["wdt"]
+            st[f"mod{method}"] = m
+        return lambda st: st[f"mod{method}"](x3)
+
+    table += [
+        ("torch.ops.flash_gemv.flag_gemv_gemv_atomic", "same op of the reference (flash_gemv.py:30-31); fp32 output, accumulate",
+         full + 2 * act_rows, lambda st: fg.flag_gemv_gemv_atomic(x, st["wg"], st["wu"], st["wdt"], out32, t)),
+        ("out.zero_() + torch.ops.flash_gemv.flag_gemv_gemv_atomic", "the same with the zero fill its contract asks of the caller",
+         full + 2 * act_rows, zeroed(lambda st: fg.flag_gemv_gemv_atomic(x, st["wg"], st["wu"], st["wdt"], out32, t))),
+        ("torch.ops.flash_gemv.fuse_gemv_gemv_gemv", "same op of the reference (flash_gemv.py:15-16); fp32 output, accumulate",
+         full + 2 * act_rows, lambda st: fg.fuse_gemv_gemv_gemv(x, st["wg"], st["wu"], st["wdt"], out32, t)),
+        ("torch.ops.flash_gemv.fuse_gemv_flag_gemv_gemv", "same op of the reference (flash_gemv.py:12-13); also writes the flags",
+         full + 2 * act_rows, lambda st: fg.fuse_gemv_flag_gemv_gemv(x, st["wg"], st["wu"], st["wdt"], out32, flag1, t)),
+        ("torch.ops.flash_gemv.flag_gemv_gemv_inner", "same op of the reference (flash_gemv.py:36-37; sp_method 1): HF-layout dense down",
+         2 * full + act_rows, lambda st: fg.flag_gemv_gemv_inner(x3, st["wg"], st["wu"], st["wd"], t)),
+        ("SiLU(x @ Wgate) + flash_gemv.gemv_gemv_triton", "the reference microbenchmark's 'Triton' column as it times it "
+         "(bench/profile_llama7B.py:16-18): torch gate GEMV and SiLU, then the sparse up / down call; this is the sp_method 2 path",
+         full + 2 * act_rows, lambda st: fg.gemv_gemv_triton(x3, act_fn(torch.matmul(x3, st["wg_t"])), st["wu"], st["wdt"], t)),
+        ("CatsMLP.forward sp_method 1", "module call (ugly_utils.py:877-886)", 2 * full + act_rows, module_call(1)),
+        ("CatsMLP.forward sp_method 2", "module call (ugly_utils.py:887-894)", full + 2 * act_rows, module_call(2)),
+        ("CatsMLP.forward sp_method 3", "module call: the whole MLP in the HIP kernels", full + 2 * act_rows, module_call(3)),
     ]
     res = []
     for name, replaces, nbytes, fn in table:

@@ -23,6 +23,7 @@ SYMBOLS = (
     "cats_version", "cats_status_string", "cats_workspace_bytes", "cats_workspace_init", "cats_gate_flag",
     "cats_gate_compact", "cats_read_count", "cats_up_flag", "cats_down_flag", "cats_gate_up", "cats_mlp",
     "cats_mlp_rowmajor_down", "cats_mlp_norm_residual", "cats_up_down", "cats_set_tuning", "cats_mlp_stage", "cats_mlp_noalloc", "cats_up_index", "cats_down_index",
+    "cats_probe_read",
 )
 
 
@@ -225,6 +226,13 @@ def mlp_rowmajor_down(x, wgate, wup, wdown, threshold, ws: Workspace):
     check(lib().cats_mlp_rowmajor_down(_p(x), _p(wgate), _p(wup), _p(wdown), _p(y), B, H, I, DTYPE_CODE[x.dtype], float(threshold),
                                        _p(ws.buf), ws.nbytes, _stream(x)), "cats_mlp_rowmajor_down")
     return y
+
+
+def probe_read(src: torch.Tensor, sink: torch.Tensor):
+    """One read-only streaming pass over src (any dtype, contiguous); sink: 4 bytes of device memory, normally untouched."""
+    fn = lib().cats_probe_read
+    fn.argtypes, fn.restype = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p], ctypes.c_int
+    check(fn(_p(src), src.numel() * src.element_size(), _p(sink), _stream(src)), "cats_probe_read")
 
 
 def set_tuning(gate_variant=0, down_groups=0, down_block=0, path=0):

@@ -65,6 +65,28 @@ __global__ void fill_zero_kernel(u32x4* p, size_t n16) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) p[i] = zero4();
 }
 
+// Read stream of known size for the measured bandwidth ceiling: every thread reads 16-byte vectors with the same
+// streaming loads the weight rows take, eight in flight, and folds them into one word that is stored only if the fold
+// hits a value the caller chooses (so the loads cannot be dropped and nothing is written otherwise).
+__global__ __launch_bounds__(1024) void read_probe_kernel(const u32x4* __restrict__ src, size_t n16, uint32_t never, uint32_t* sink) {
+  constexpr int U = 8;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  uint32_t acc = 0;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i + (U - 1) * stride < n16; i += U * stride) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = load_stream(src + i + u * stride);
+#pragma unroll
+    for (int u = 0; u < U; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  for (; i < n16; i += stride) {
+    const u32x4 v = load_stream(src + i);
+    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+  }
+  if (acc == never) *sink = acc;
+}
+
 // Number of neurons flagged in any of the B rows of flags (B, I): the count of a call that ran as several passes.
 __global__ __launch_bounds__(1024) void union_count_kernel(const uint8_t* __restrict__ flags, int B, int I, int32_t* count_out) {
   __shared__ int s_part[16];
@@ -489,6 +511,15 @@ int cats_gate_compact(const void* x, const void* wgate, void* vals_out, int64_t*
   const hipError_t e = elem_size(dtype) == 2 ? launch_kernel(compact_kernel<2>, dim3(groups), dim3(256), 0, (hipStream_t)stream, c)
                                              : launch_kernel(compact_kernel<4>, dim3(groups), dim3(256), 0, (hipStream_t)stream, c);
   return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+}
+
+int cats_probe_read(const void* src, size_t bytes, uint32_t* sink, void* stream) {
+  if (!src || !sink) return CATS_ERR_NULL;
+  if (!aligned16(src) || bytes % 16 != 0 || bytes == 0) return CATS_ERR_ALIGN;
+  const int grid = current_device_cus() * 2;
+  return launch_kernel(read_probe_kernel, dim3(grid), dim3(1024), 0, (hipStream_t)stream, (const u32x4*)src, bytes / 16, 0x9e3779b9u, sink) == hipSuccess
+             ? CATS_OK
+             : CATS_ERR_LAUNCH;
 }
 
 int cats_read_count(const int32_t* count_dev, void* stream) {

@@ -163,7 +163,9 @@ struct FusedSlots {
 // The wave looks at 64 slots per pass -- lane i reads state and z of slot head + i, ballots find the decided prefix and
 // the kept slots in it -- so a pass costs one LDS round trip however many dead slots it steps over.
 // n: the caller's copy of the number of slots in use, refreshed here.
-template <int B, int KV, int RB>
+// ANN false: an announced slot counts as pending (the wave holds too many registers of row data to also carry the
+// bookkeeping of rows whose z is still to come).
+template <int B, int KV, int RB, bool ANN>
 __device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const FusedSlots& sl, int& head, int& n, bool blocking) {
   bt.cnt = 0;
   bt.unresolved = 0;
@@ -182,9 +184,9 @@ __device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const Fu
     if (kFusedPool) n = __builtin_amdgcn_readfirstlane(__hip_atomic_load(sl.nfinal, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
     if (head >= n) return;
     if (idx >= n) st_ = kSlotPending;  // slots past the last one in use may never have been written
-    const uint64_t pend = __ballot(st_ == kSlotPending);
-    uint64_t live = __ballot(st_ >= kSlotAnnounced);
-    const uint64_t hasz = __ballot(st_ == kSlotLive);
+    const uint64_t pend = __ballot(ANN ? st_ == kSlotPending : (st_ == kSlotPending || st_ == kSlotAnnounced));
+    uint64_t live = __ballot(ANN ? st_ >= kSlotAnnounced : st_ == kSlotLive);
+    const uint64_t hasz = ANN ? __ballot(st_ == kSlotLive) : ~0ull;
     const int ready = pend ? __builtin_ctzll(pend) : kWave;  // slots head .. head + ready - 1 are decided
     if (ready == 0) {
       if (!blocking) return;
@@ -204,8 +206,8 @@ __device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const Fu
         const int bit = __builtin_ctzll(live);
         live &= live - 1ull;
         bt.rows[u] = __builtin_amdgcn_readlane(rowv, bit);
-        bt.slots[u] = head + bit;
-        if ((hasz >> bit) & 1ull) {
+        if (ANN) bt.slots[u] = head + bit;
+        if (!ANN || ((hasz >> bit) & 1ull)) {
 #pragma unroll
           for (int b = 0; b < B; b++) bt.zz[u][b] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(zv[b], bit));
         } else {
@@ -222,9 +224,9 @@ __device__ __forceinline__ void fused_collect(DownBatch<B, KV, RB>& bt, const Fu
 
 // Wait until the z of every row of the batch is in its slot, and read those that fused_collect could not.  Lane u
 // watches row u.
-template <int B, int KV, int RB>
+template <int B, int KV, int RB, bool ANN>
 __device__ __forceinline__ void fused_resolve(DownBatch<B, KV, RB>& bt, const FusedSlots& sl) {
-  if (bt.unresolved == 0) return;  // uniform
+  if (!ANN || bt.unresolved == 0) return;  // uniform
   const int lane = threadIdx.x & (kWave - 1);
   int myslot = -1;
 #pragma unroll
@@ -282,6 +284,7 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   constexpr int VEC = DT::VEC;
   constexpr int RW = kFusedWaves - DW;
   constexpr int RB = 8 / (KV * B) < 1 ? 1 : 8 / (KV * B);  // row slots per batch of a down wave; two batches are in flight
+  constexpr bool ANN = true;  // down waves send for a row as soon as its neuron is known to be kept (see fused_collect)
   constexpr int kXPre = 2;  // x vectors per thread fetched ahead of the first weight block
   extern __shared__ u32x4 s_fused[];
   __shared__ int s_ticket;
@@ -650,34 +653,38 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
   int head = 0, nlive = 0;
   int nfin = kFusedPool ? p.cap : n;  // slots in use, as far as this wave knows (the pool build refreshes it in fused_collect)
   DownBatch<B, KV, RB> ba, bb;
-  fused_collect<B, KV, RB>(ba, sl, head, nfin, true);
+  // TAIL: when nothing is left to send for, finish the batch in flight and leave no load behind (whatever is still
+  // outstanding when the sums are written out has to be waited for first).  Worth half a microsecond on rows of up to
+  // 2 * DW * 64 vectors; with four vectors per lane per row the extra exits cost registers the wave does not have
+  // (spills), so there the last round issues its (cached, unused) loads like any other.
+  constexpr bool TAIL = KV < 4;
+  fused_collect<B, KV, RB, ANN>(ba, sl, head, nfin, true);
   fused_down_issue<B, KV, RB>(ba, p.wd, p.row_vecs, p.x, vidx);
   for (;;) {
     if (ba.cnt == 0 && head >= nfin) break;
-    fused_collect<B, KV, RB>(bb, sl, head, nfin, ba.cnt == 0);
-    if (bb.cnt == 0 && head >= nfin) {
-      // nothing left to send for: finish the batch in flight and leave no load behind (whatever is still outstanding
-      // when the sums are written out has to be waited for first)
-      fused_resolve<B, KV, RB>(ba, sl);
+    fused_collect<B, KV, RB, ANN>(bb, sl, head, nfin, ba.cnt == 0);
+    if (TAIL && bb.cnt == 0 && head >= nfin) {
+      fused_resolve<B, KV, RB, ANN>(ba, sl);
       fused_down_consume<DT, B, KV, RB>(ba, acc);
       nlive += ba.cnt;
       break;
     }
     CATS_FSTAMP(lane == 0 && d == 0 && bb.cnt > 0, 5);
     fused_down_issue<B, KV, RB>(bb, p.wd, p.row_vecs, p.x, vidx);
-    fused_resolve<B, KV, RB>(ba, sl);
+    fused_resolve<B, KV, RB, ANN>(ba, sl);
     fused_down_consume<DT, B, KV, RB>(ba, acc);
     nlive += ba.cnt;
-    fused_collect<B, KV, RB>(ba, sl, head, nfin, bb.cnt == 0);
-    if (ba.cnt == 0 && head >= nfin) {
-      fused_resolve<B, KV, RB>(bb, sl);
+    if (!TAIL && bb.cnt == 0 && head >= nfin) break;
+    fused_collect<B, KV, RB, ANN>(ba, sl, head, nfin, bb.cnt == 0);
+    if (TAIL && ba.cnt == 0 && head >= nfin) {
+      fused_resolve<B, KV, RB, ANN>(bb, sl);
       fused_down_consume<DT, B, KV, RB>(bb, acc);
       nlive += bb.cnt;
       break;
     }
     CATS_FSTAMP(lane == 0 && d == 0 && ba.cnt > 0, 5);
     fused_down_issue<B, KV, RB>(ba, p.wd, p.row_vecs, p.x, vidx);
-    fused_resolve<B, KV, RB>(bb, sl);
+    fused_resolve<B, KV, RB, ANN>(bb, sl);
     fused_down_consume<DT, B, KV, RB>(bb, acc);
     nlive += bb.cnt;
   }

@@ -193,6 +193,13 @@ int cats_mlp_noalloc(const void* x, const void* wgate, const void* wup, const vo
 int cats_mlp_stage(int stage, const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out,
                    int B, int H, int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream);
 
+/* Measurement aid, not in the reference: one kernel that reads `bytes` (a multiple of 16, 16-byte aligned) from src
+ * with the streaming 128-bit loads the weight rows are read with, and writes nothing (sink, 4 bytes of device memory,
+ * is stored to only if the XOR of everything read equals one fixed word).  Timing it over a buffer larger than the
+ * 256 MB memory-side cache gives the read-stream bandwidth this GPU actually reaches, the practical ceiling next
+ * to the published HBM peak. */
+int cats_probe_read(const void* src, size_t bytes, uint32_t* sink, void* stream);
+
 /* Launch-shape knobs for experiments; 0 keeps the built-in choice.  gate_variant N > 0 caps the gate / up kernel at N
  * resident workgroups per CU (N < 0 keeps 3..8 rows off the matrix-core kernel); down_groups / down_block set the neuron
  * groups and the workgroup size of the sparse down kernel; path 1 keeps the whole-MLP entry points on the separate gate+up
