@@ -568,6 +568,8 @@ def entry_points(torch, F, capi, steps, warmup, only=()):
          full + 2 * act_rows, lambda st: capi.mlp(x, st["wg"], st["wu"], st["wdt"], t, ws, y_f32=out32)),
         ("cats_mlp_norm_residual", "norm -> mlp -> residual of the decoder layer", full + 2 * act_rows,
          lambda st: capi.mlp_norm_residual(x, nw, 1e-5, st["wg"], st["wu"], st["wdt"], t, ws)),
+        ("cats_mlp_norm_residual_norm", "the same plus the next layer's input norm from the finishing launch", full + 2 * act_rows,
+         lambda st: capi.mlp_norm_residual_norm(x, nw, 1e-5, st["wg"], st["wu"], st["wdt"], t, nw, 1e-5, ws)),
         ("cats_mlp_rowmajor_down", "flag_gemv_gemv, flag_gemv_gemv_inner*", 2 * full + act_rows, lambda st: capi.mlp_rowmajor_down(x, st["wg"], st["wu"], st["wd"], t, ws)),
     ]
     # the registered torch ops and the Python composites, called as a user of the reference's package calls them

@@ -23,7 +23,7 @@ SYMBOLS = (
     "cats_version", "cats_status_string", "cats_workspace_bytes", "cats_workspace_init", "cats_gate_flag",
     "cats_gate_compact", "cats_read_count", "cats_up_flag", "cats_down_flag", "cats_gate_up", "cats_mlp",
     "cats_mlp_rowmajor_down", "cats_mlp_norm_residual", "cats_up_down", "cats_set_tuning", "cats_mlp_stage", "cats_mlp_noalloc", "cats_up_index", "cats_down_index",
-    "cats_probe_read",
+    "cats_probe_read", "cats_mlp_norm_residual_norm",
 )
 
 
@@ -60,6 +60,9 @@ def lib() -> ctypes.CDLL:
         L.cats_mlp_rowmajor_down.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_mlp_rowmajor_down.restype = i32
         L.cats_mlp_norm_residual.argtypes = [vp, vp, f32, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]
         L.cats_mlp_norm_residual.restype = i32
+        if hasattr(L, "cats_mlp_norm_residual_norm"):  # absent from older builds of the library bound with use_library()
+            L.cats_mlp_norm_residual_norm.argtypes = [vp, vp, f32, vp, vp, vp, vp, vp, f32, vp, i32, i32, i32, i32, f32, vp, sz, vp]
+            L.cats_mlp_norm_residual_norm.restype = i32
         L.cats_up_down.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_up_down.restype = i32
         L.cats_mlp_stage.argtypes = [i32, vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, sz, vp]; L.cats_mlp_stage.restype = i32
         L.cats_mlp_noalloc.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp]; L.cats_mlp_noalloc.restype = i32
@@ -218,6 +221,18 @@ def mlp_norm_residual(h, norm_weight, eps, wgate, wup, wdown_t, threshold, ws: W
                                        DTYPE_CODE[h.dtype], float(threshold), _p(ws.buf), ws.nbytes, _stream(h)),
           "cats_mlp_norm_residual")
     return out
+
+
+def mlp_norm_residual_norm(h, norm_weight, eps, wgate, wup, wdown_t, threshold, next_norm_weight, next_eps, ws: Workspace, out=None):
+    """(out, next_out): out = h + MLP(norm_weight * rms_norm(h)), next_out = next_norm_weight * rms_norm(out)."""
+    B, H, I = _dims(h, wgate)
+    if out is None:
+        out = torch.empty(B, H, dtype=h.dtype, device=h.device)
+    nxt = torch.empty(B, H, dtype=h.dtype, device=h.device)
+    check(lib().cats_mlp_norm_residual_norm(_p(h), _p(norm_weight), float(eps), _p(wgate), _p(wup), _p(wdown_t), _p(out),
+                                            _p(next_norm_weight), float(next_eps), _p(nxt), B, H, I, DTYPE_CODE[h.dtype],
+                                            float(threshold), _p(ws.buf), ws.nbytes, _stream(h)), "cats_mlp_norm_residual_norm")
+    return out, nxt
 
 
 def mlp_rowmajor_down(x, wgate, wup, wdown, threshold, ws: Workspace):

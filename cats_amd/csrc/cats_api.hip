@@ -53,9 +53,15 @@ long long* g_tbuf_fused = nullptr;
 
 constexpr int kMaxSlabs = 128;
 constexpr int kKernelBatch = 8;  // rows one launch handles; the entry points take up to CATS_MAX_BATCH rows in passes of this many
-// Head of the workspace: the neuron-pool counters of the single-pass kernel (one 128-byte line per group of workgroups).
-// Zeroed by cats_workspace_init and put back to zero by every call that uses them.
-constexpr size_t kCounterBytes = 1024 + 64 * 128;
+// Head of the workspace.  [0, 4096): the neuron-pool counters of the single-pass kernel (one 128-byte line per group of
+// workgroups; pool builds only).  then the arrival counters of the reduction launch that also writes the next norm
+// (72 lines of 128 bytes).  Both are zeroed by cats_workspace_init and put back to zero by every call that uses them.
+// Last: the per-workgroup sums of squares of that launch (overwritten by every call).
+constexpr size_t kPoolCounterBytes = 4096;
+constexpr size_t kArriveOffset = kPoolCounterBytes;
+constexpr size_t kSsqOffset = kArriveOffset + (size_t)(8 * kArriveGroups + 8) * kArriveStride * 4;
+constexpr size_t kSsqFloats = 4096;  // workgroups of the reduction launch: B * H / 32
+constexpr size_t kCounterBytes = kSsqOffset + kSsqFloats * 4;
 #ifndef CATS_POOL_NUM  // share of a workgroup's neurons that goes to its group's pool (builds with -DCATS_FUSED_POOL=1 only)
 #define CATS_POOL_NUM 1
 #define CATS_POOL_DEN 4
@@ -65,22 +71,25 @@ __global__ void fill_zero_kernel(u32x4* p, size_t n16) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) p[i] = zero4();
 }
 
-// Read stream of known size for the measured bandwidth ceiling: every thread reads 16-byte vectors with the same
-// streaming loads the weight rows take, eight in flight, and folds them into one word that is stored only if the fold
-// hits a value the caller chooses (so the loads cannot be dropped and nothing is written otherwise).
-__global__ __launch_bounds__(1024) void read_probe_kernel(const u32x4* __restrict__ src, size_t n16, uint32_t never, uint32_t* sink) {
+// Read stream of known size for the measured bandwidth ceiling: every workgroup walks its own contiguous span (the
+// fastest of the shapes tried: 7.0 TB/s on the MI355X against 6.7 for a grid-strided walk), every thread reads 16-byte
+// vectors with the same streaming loads the weight rows take, eight in flight, and folds them into one word that is
+// stored only if the fold hits a value the caller chooses (so the loads cannot be dropped and nothing is written).
+__global__ __launch_bounds__(512) void read_probe_kernel(const u32x4* __restrict__ src, size_t n16, uint32_t never, uint32_t* sink) {
   constexpr int U = 8;
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const size_t span = (n16 + gridDim.x - 1) / gridDim.x;
+  const size_t lo = (size_t)blockIdx.x * span < n16 ? (size_t)blockIdx.x * span : n16;
+  const size_t hi = lo + span < n16 ? lo + span : n16;
   uint32_t acc = 0;
-  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  for (; i + (U - 1) * stride < n16; i += U * stride) {
+  size_t i = lo + threadIdx.x;
+  for (; i + (size_t)(U - 1) * blockDim.x < hi; i += (size_t)U * blockDim.x) {
     u32x4 v[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) v[u] = load_stream(src + i + u * stride);
+    for (int u = 0; u < U; u++) v[u] = load_stream(src + i + (size_t)u * blockDim.x);
 #pragma unroll
     for (int u = 0; u < U; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
   }
-  for (; i < n16; i += stride) {
+  for (; i < hi; i += blockDim.x) {
     const u32x4 v = load_stream(src + i);
     acc ^= v.x ^ v.y ^ v.z ^ v.w;
   }
@@ -110,7 +119,7 @@ __global__ __launch_bounds__(1024) void union_count_kernel(const uint8_t* __rest
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct WsLayout {
-  size_t counters, mask, z32, zt, partial, atmp, total;
+  size_t counters, mask, z32, zt, partial, atmp, fin, total;
 };
 
 constexpr int kMaxGroups = 64;  // neuron groups of the sparse down kernel; bounds the partial-sum scratch
@@ -127,6 +136,7 @@ WsLayout ws_layout(int H, int I) {
   l.z32 = o;      o += align_up((size_t)B * I * 4, 256);
   l.zt = o;       o += align_up((size_t)B * I * 4, 256);
   l.atmp = o;     o += align_up((size_t)B * I * 4, 256);
+  l.fin = o;      o += align_up((size_t)B * H * 4, 256);  // finished columns as fp32, for the launch that also writes the next norm
   l.total = o;
   return l;
 }
@@ -233,10 +243,30 @@ int do_rows(int mode, int dtype, const RowsArgs& a_in, hipStream_t s) {
   return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
 }
 
+// Optional second output of the launch that finishes y: next.out = next.w * rms_norm(y).
+struct NextNorm {
+  const void* w = nullptr;
+  float eps = 0.f;
+  void* out = nullptr;
+};
+
+// Fills the next-norm fields of the reduction launch; CATS_ERR_SHAPE if the launch cannot carry it.
+int set_next_norm(ReduceArgs& r, const NextNorm& next, char* ws, const WsLayout& l) {
+  if (!next.out) return CATS_OK;
+  if (r.H % kReduceCols != 0 || (size_t)(r.BH / kReduceCols) > kSsqFloats) return CATS_ERR_SHAPE;
+  r.norm2_out = next.out;
+  r.norm2_w = next.w;
+  r.norm2_eps = next.eps;
+  r.arrive = (int32_t*)(ws + l.counters + kArriveOffset);
+  r.ssq_part = (float*)(ws + l.counters + kSsqOffset);
+  r.fin = (float*)(ws + l.fin);
+  return CATS_OK;
+}
+
 // Sparse down over mask words already in the workspace.
 int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_out, int32_t* count_out, int B, int H, int I,
             int dtype, char* ws, const WsLayout& l, hipStream_t s, const void* residual = nullptr, const uint8_t* flags = nullptr,
-            const int64_t* idx = nullptr, int M = 0, const void* bias = nullptr) {
+            const int64_t* idx = nullptr, int M = 0, const void* bias = nullptr, const NextNorm& next = NextNorm()) {
   DownArgs d;
   memset(&d, 0, sizeof(d));
   d.wd = (const u32x4*)wdown_t;
@@ -285,6 +315,7 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   r.H = H;
   r.G = d.ngroup;
   r.BH = B * H;
+  if (int st = set_next_norm(r, next, ws, l)) return st;
   FusedArgs none;
   memset(&none, 0, sizeof(none));
   if (dtype == CATS_F16) e = launch_fused<F16>(1, 0, 2, none, r, s);
@@ -345,11 +376,11 @@ void fused_enable_pool(FusedArgs& f, int grid, int dtype, int32_t* counters, siz
 // y32 set: the streaming kernel adds into the caller's fp32 accumulator itself and nothing is launched after it,
 // unless the caller wants the count of active neurons (then the second launch does only that).
 int do_fused(FusedArgs& f, int grid, int stage, void* y_out, const void* residual, int32_t* count_out, int dtype, char* ws,
-             const WsLayout& l, hipStream_t s, float* y32 = nullptr) {
+             const WsLayout& l, hipStream_t s, float* y32 = nullptr, const NextNorm& next = NextNorm()) {
   f.partial = (float*)(ws + l.partial);
   f.counts = (int32_t*)(ws + l.z32);
   f.y32 = y32;
-  fused_enable_pool(f, grid, dtype, (int32_t*)(ws + l.counters), kCounterBytes);
+  fused_enable_pool(f, grid, dtype, (int32_t*)(ws + l.counters), kPoolCounterBytes);
 #ifdef CATS_TIMING
   f.tbuf = g_tbuf_fused;
 #endif
@@ -367,6 +398,7 @@ int do_fused(FusedArgs& f, int grid, int stage, void* y_out, const void* residua
     r.BH = 0;  // no columns to finish
     if (stage == 0 && !count_out) stage = 1;
   }
+  if (int st = set_next_norm(r, next, ws, l)) return st;
   const int bt = batch_template(f.nb);
   hipError_t e;
   if (dtype == CATS_F16) e = launch_fused<F16>(bt, grid, stage, f, r, s);
@@ -516,8 +548,8 @@ int cats_gate_compact(const void* x, const void* wgate, void* vals_out, int64_t*
 int cats_probe_read(const void* src, size_t bytes, uint32_t* sink, void* stream) {
   if (!src || !sink) return CATS_ERR_NULL;
   if (!aligned16(src) || bytes % 16 != 0 || bytes == 0) return CATS_ERR_ALIGN;
-  const int grid = current_device_cus() * 2;
-  return launch_kernel(read_probe_kernel, dim3(grid), dim3(1024), 0, (hipStream_t)stream, (const u32x4*)src, bytes / 16, 0x9e3779b9u, sink) == hipSuccess
+  const int grid = current_device_cus() * 4;
+  return launch_kernel(read_probe_kernel, dim3(grid), dim3(512), 0, (hipStream_t)stream, (const u32x4*)src, bytes / 16, 0x9e3779b9u, sink) == hipSuccess
              ? CATS_OK
              : CATS_ERR_LAUNCH;
 }
@@ -652,7 +684,7 @@ static int up_down_pass(const void* x, const void* a_in, const void* wup, const 
 
 static int mlp_norm_residual_pass(const void* h, const void* norm_weight, float eps, const void* wgate, const void* wup,
                            const void* wdown_t, void* out, int B, int H, int I, int dtype, float threshold, void* ws,
-                           size_t ws_bytes, void* stream) {
+                           size_t ws_bytes, void* stream, const NextNorm& next = NextNorm()) {
   int st = check_common(B, H, I, dtype);
   if (st) return st;
   if (!h || !norm_weight || !wgate || !wup || !wdown_t || !out) return CATS_ERR_NULL;
@@ -672,7 +704,7 @@ static int mlp_norm_residual_pass(const void* h, const void* norm_weight, float 
     f.t = round_through(dtype, threshold);
     f.norm_w = (const u32x4*)norm_weight;
     f.norm_eps = eps;
-    return do_fused(f, grid, 0, out, h, nullptr, dtype, (char*)ws, l, (hipStream_t)stream);
+    return do_fused(f, grid, 0, out, h, nullptr, dtype, (char*)ws, l, (hipStream_t)stream, nullptr, next);
   }
   RowsArgs a;
   fill_rows(a, h, wgate, H, I, B, dtype);
@@ -684,7 +716,8 @@ static int mlp_norm_residual_pass(const void* h, const void* norm_weight, float 
   a.norm_eps = eps;
   st = do_rows(kGateUp, dtype, a, (hipStream_t)stream);
   if (st) return st;
-  return do_down(a.z32_out, true, wdown_t, nullptr, out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream, h);
+  return do_down(a.z32_out, true, wdown_t, nullptr, out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream, h, nullptr, nullptr, 0,
+                 nullptr, next);
 }
 
 static int mlp_rowmajor_down_pass(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out, int B, int H,
@@ -886,6 +919,23 @@ int cats_mlp_norm_residual(const void* h, const void* norm_weight, float eps, co
   return in_passes(B, [&](size_t b0, int nb) {
     return mlp_norm_residual_pass(at_cbytes(h, b0 * H * sz), norm_weight, eps, wgate, wup, wdown_t, at_bytes(out, b0 * H * sz), nb, H, I, dtype,
                                   threshold, ws, ws_bytes, stream);
+  });
+}
+
+int cats_mlp_norm_residual_norm(const void* h, const void* norm_weight, float eps, const void* wgate, const void* wup,
+                                const void* wdown_t, void* out, const void* next_norm_weight, float next_eps, void* next_out, int B,
+                                int H, int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
+  if (!next_norm_weight || !next_out) return CATS_ERR_NULL;
+  if (!aligned16(next_norm_weight) || !aligned16(next_out)) return CATS_ERR_ALIGN;
+  if (H % kReduceCols != 0) return CATS_ERR_SHAPE;
+  const size_t sz = esz(dtype);
+  return in_passes(B, [&](size_t b0, int nb) {
+    NextNorm next;
+    next.w = next_norm_weight;
+    next.eps = next_eps;
+    next.out = at_bytes(next_out, b0 * H * sz);
+    return mlp_norm_residual_pass(at_cbytes(h, b0 * H * sz), norm_weight, eps, wgate, wup, wdown_t, at_bytes(out, b0 * H * sz), nb, H, I, dtype,
+                                  threshold, ws, ws_bytes, stream, next);
   });
 }
 

@@ -44,6 +44,8 @@ constexpr int kFusedMaxKV = 4;          // a down wave covers KV * 64 vectors of
 constexpr bool kFusedPool = CATS_FUSED_POOL != 0;
 constexpr int kFusedGroup = 8;          // consecutive workgroups (one per XCD) that share a pool of neurons
 constexpr int kPoolStride = 32;         // int32 per group in the pool counter array: ticket counter at +0, finished workgroups at +16
+constexpr int kArriveGroups = 8;        // groups a batch row's workgroups of the reduction launch arrive in
+constexpr int kArriveStride = 32;       // int32 between arrival counters: one 128-byte line each
 constexpr int kReduceCols = 32;         // fp32 columns per workgroup of the reduction kernel
 constexpr int kReduceLanes = 32;        // ranges of partials summed side by side per column
 
@@ -103,6 +105,14 @@ struct ReduceArgs {
   int32_t* count_out;    // optional
   int G;                 // number of partials
   int BH;                // nb * H
+  // optional second output: norm2_out (nb, H) dtype = norm2_w * rms_norm(y_out) -- the norm the next consumer of the
+  // hidden state starts with.  Needs H % kReduceCols == 0 (a workgroup's columns lie in one row).
+  void* norm2_out;
+  const void* norm2_w;   // (H,) dtype
+  float norm2_eps;
+  float* ssq_part;       // [gridDim] sum of squares of every workgroup's columns
+  float* fin;            // [BH] the finished columns as fp32, for the workgroup that writes norm2_out
+  int32_t* arrive;       // arrival counters, zero between calls: [8 rows][kArriveGroups] then [8 rows], kArriveStride apart
 };
 
 #ifdef CATS_TIMING
@@ -797,6 +807,100 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(ReduceArgs p) {
       if (p.bias) tot += DT::tof(((const st*)p.bias)[c % p.H]);
       if (p.residual) tot = DT::rnd(tot) + DT::tof(((const st*)p.residual)[c]);
       ((st*)p.y_out)[c] = DT::fromf(tot);
+    }
+  }
+  if (p.norm2_out) {
+    // The norm of the finished rows needs every column's square.  Each workgroup leaves its finished columns (as fp32, the
+    // values as stored, i.e. rounded to the storage type) and the sum of their squares in the workspace; the workgroup
+    // that finds itself the last to arrive adds the sums per row in workgroup order -- a fixed order, so the result
+    // does not vary from run to run -- and writes the normalised rows.
+    // What the other workgroups leave for that one is written with device-scope atomic stores (they write through to
+    // the level all XCDs share) and the wave waits for them to be acknowledged before its arrival is counted; the last
+    // workgroup invalidates its caches once (acquire fence) and reads with plain vector loads.  A device-scope release
+    // fence in every workgroup would order plain stores the same way, but it writes back the whole L2 each time.
+    __shared__ int s_last;
+    __shared__ float s_scale2;
+    const int wpr = p.H / kReduceCols;   // workgroups per row
+    const int brow = blockIdx.x / wpr;   // the batch row this workgroup's columns belong to (H % kReduceCols == 0)
+    if (tid < kWave) {
+      float v = 0.f;
+      const int c = blockIdx.x * kReduceCols + tid;
+      if (tid < kReduceCols && c < p.BH) {
+        v = DT::tof(((const st*)p.y_out)[c]);  // this thread's own store, just above
+        __hip_atomic_store(&p.fin[c], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      v = wave_sum(v * v);
+      if (tid == 0) __hip_atomic_store(&p.ssq_part[blockIdx.x], v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_s_waitcnt(0);  // every store of this wave has been acknowledged
+      // Arrivals are counted per batch row (the rows are finished by different workgroups, side by side) and in two
+      // levels, every counter in a cache line of its own: atomics on one line take their turns (12 ns each on the
+      // MI355X), so 1024 workgroups on one line would queue for 12 us.  A row's workgroups form up to kArriveGroups
+      // groups; the last of a group reports the group to the row's counter.
+      if (tid == 0) {
+        const int gsize = (wpr + kArriveGroups - 1) / kArriveGroups;
+        const int wi = blockIdx.x - brow * wpr, g = wi / gsize;
+        const int members = min(gsize, wpr - g * gsize), ngroups = (wpr + gsize - 1) / gsize;
+        int32_t* c1 = p.arrive + (size_t)(brow * kArriveGroups + g) * kArriveStride;
+        int32_t* c2 = p.arrive + (size_t)(8 * kArriveGroups + brow) * kArriveStride;
+        int last = 0;
+        if (__hip_atomic_fetch_add(c1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1) {
+          __hip_atomic_store(c1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // nobody else comes to this counter in this call
+          if (__hip_atomic_fetch_add(c2, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ngroups - 1) {
+            __hip_atomic_store(c2, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last = 1;
+          }
+        }
+        s_last = last;
+      }
+    }
+    __syncthreads();
+    if (s_last) {  // uniform
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      if (tid < kWave) {
+        float ss = 0.f;
+        for (int w = tid; w < wpr; w += kWave) ss += p.ssq_part[brow * wpr + w];
+        ss = wave_sum(ss);
+        if (tid == 0) s_scale2 = rsqrtf(ss / (float)p.H + p.norm2_eps);
+      }
+      __syncthreads();
+      constexpr int VEC = DT::VEC;
+      constexpr int U = 2;  // vectors per thread whose loads go out together
+      const int row_vecs = p.H / VEC;
+      const float4* f4 = (const float4*)(p.fin + (size_t)brow * p.H);
+      const u32x4* w4 = (const u32x4*)p.norm2_w;
+      u32x4* o4 = (u32x4*)p.norm2_out + (size_t)brow * row_vecs;
+      const float sc = s_scale2;
+      for (int v0 = tid; v0 < row_vecs; v0 += U * 256) {
+        float4 x4[U][VEC / 4];
+        u32x4 wv[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          const int v = min(v0 + u * 256, row_vecs - 1);
+#pragma unroll
+          for (int q = 0; q < VEC / 4; q++) x4[u][q] = f4[(size_t)v * (VEC / 4) + q];
+          wv[u] = w4[v];
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          const int v = v0 + u * 256;
+          if (v < row_vecs) {
+            // the finished values are exact in the storage type: packed back, the norm is the same routine the staging
+            // of x uses (weight * round(x * scale), both roundings through the storage type)
+            u32x4 xv;
+            if constexpr (sizeof(st) == 4) {
+              xv[0] = __float_as_uint(x4[u][0].x); xv[1] = __float_as_uint(x4[u][0].y);
+              xv[2] = __float_as_uint(x4[u][0].z); xv[3] = __float_as_uint(x4[u][0].w);
+            } else {
+#pragma unroll
+              for (int q = 0; q < VEC / 4; q++) {
+                xv[2 * q] = (uint32_t)DT::fromf(x4[u][q].x) | ((uint32_t)DT::fromf(x4[u][q].y) << 16);
+                xv[2 * q + 1] = (uint32_t)DT::fromf(x4[u][q].z) | ((uint32_t)DT::fromf(x4[u][q].w) << 16);
+              }
+            }
+            o4[v] = vec_norm_apply<DT>(xv, sc, wv[u]);
+          }
+        }
+      }
     }
   }
   if (p.count_out && blockIdx.x == 0 && tid >= 64 && tid < 128) {  // second wave: total of the per-workgroup counts

@@ -405,6 +405,32 @@ at::Tensor cats_mlp_norm_residual_op(const at::Tensor& h, const at::Tensor& norm
   return out;
 }
 
+// (out, next) with out as above and next = next_norm_weight * rms_norm(out, next_eps): the norm the following layer starts with.
+std::tuple<at::Tensor, at::Tensor> cats_mlp_norm_residual_norm_op(const at::Tensor& h, const at::Tensor& norm_weight, const double eps,
+                                                                  const at::Tensor& wgate, const at::Tensor& wup, const at::Tensor& wdown_t,
+                                                                  const double threshold, const at::Tensor& next_norm_weight,
+                                                                  const double next_eps) {
+  check_dev(h, "h");
+  const int B = batch_rows(h, "cats_mlp_norm_residual_norm");
+  const int64_t H = h.size(-1), I = wgate.size(0);
+  check_weight(wgate, h, I, H, "wgate");
+  check_weight(wup, h, I, H, "wup");
+  check_weight(wdown_t, h, I, H, "wdown_t (neuron-major)");
+  for (const at::Tensor* w : {&norm_weight, &next_norm_weight})
+    TORCH_CHECK(w->is_cuda() && w->is_contiguous() && w->scalar_type() == h.scalar_type() && w->numel() == H &&
+                    w->get_device() == h.get_device(),
+                "flash_gemv.cats_mlp_norm_residual_norm: the norm weights must be contiguous (H,) tensors of h's dtype on h's device");
+  at::Tensor out = at::empty_like(h);
+  at::Tensor next = at::empty_like(h);
+  hipStream_t s = current_stream(h);
+  Workspace& ws = workspace(h, B, (int)H, (int)I, s);
+  check_status(cats_mlp_norm_residual_norm(h.data_ptr(), norm_weight.data_ptr(), (float)eps, wgate.data_ptr(), wup.data_ptr(),
+                                           wdown_t.data_ptr(), out.data_ptr(), next_norm_weight.data_ptr(), (float)next_eps, next.data_ptr(),
+                                           B, (int)H, (int)I, dtype_code(h), (float)threshold, ws.buf.data_ptr(), ws.bytes, s),
+               "cats_mlp_norm_residual_norm");
+  return {out, next};
+}
+
 // Same, also returning the per-row flags (B*I bool) and the number of neurons fetched (int32 scalar tensor).
 std::tuple<at::Tensor, at::Tensor, at::Tensor> cats_mlp_stats_op(const at::Tensor& x, const at::Tensor& wgate, const at::Tensor& wup,
                                                                  const at::Tensor& wdown_t, const double threshold) {
@@ -449,6 +475,7 @@ TORCH_LIBRARY(flash_gemv, m) {
   m.def("cats_down_index", cats_down_index_op);
   m.def("cats_mlp", cats_mlp_op);
   m.def("cats_mlp_norm_residual", cats_mlp_norm_residual_op);
+  m.def("cats_mlp_norm_residual_norm", cats_mlp_norm_residual_norm_op);
   m.def("cats_up_down", cats_up_down_op);
   m.def("cats_mlp_stats", cats_mlp_stats_op);
 }

@@ -97,11 +97,18 @@ class DecoderLayer(nn.Module):
         self.post_attention_layernorm = RMSNorm(cfg.hidden_size, cfg.rms_eps, dtype, device)
         self.mlp = CatsMLP(cfg.hidden_size, cfg.intermediate_size, dtype=dtype, device=device)
         self.fuse_norm_residual = False  # decode only: post-attention norm and residual inside the two MLP launches
+        self.fuse_next_norm = False      # and the norm the next layer starts with written by the same launches
 
-    def forward(self, h, cos, sin, positions, mask):
-        h = h + self.self_attn(self.input_layernorm(h), cos, sin, positions, mask)
+    def forward(self, h, cos, sin, positions, mask, normed=None, next_norm=None):
+        """normed: input_layernorm(h) if the previous layer's MLP launches already wrote it.  next_norm: the RMSNorm
+        module that will consume this layer's output; with fuse_next_norm the return value is (h, next_norm(h))."""
+        if normed is None:
+            normed = self.input_layernorm(h)
+        h = h + self.self_attn(normed, cos, sin, positions, mask)
         if self.fuse_norm_residual and h.shape[1] == 1 and self.mlp.is_profile and self.mlp.sp_method == 3:
             n = self.post_attention_layernorm
+            if self.fuse_next_norm and next_norm is not None:
+                return self.mlp.forward_norm_residual_norm(h, n.weight, n.eps, next_norm.weight, next_norm.eps)
             return self.mlp.forward_norm_residual(h, n.weight, n.eps)
         return h + self.mlp(self.post_attention_layernorm(h))
 
@@ -140,19 +147,25 @@ class LlamaDecoder(nn.Module):
         slots = torch.arange(cfg.max_len, device=tokens.device)
         mask = torch.zeros(positions.numel(), cfg.max_len, dtype=self.dtype, device=tokens.device)
         mask.masked_fill_(slots[None, :] > positions[:, None], float("-inf"))
-        for layer in self.layers:
-            h = layer(h, cos, sin, positions, mask)
-        return self.lm_head(self.norm(h))
+        normed = None
+        for i, layer in enumerate(self.layers):
+            next_norm = self.layers[i + 1].input_layernorm if i + 1 < len(self.layers) else self.norm
+            out = layer(h, cos, sin, positions, mask, normed, next_norm)
+            h, normed = out if isinstance(out, tuple) else (out, None)
+        return self.lm_head(normed if normed is not None else self.norm(h))
 
     # ---- MLP mode switches ----
     def set_mlp_mode(self, mode: str):
         """"dense": plain SwiGLU.  "cats_torch": dense-masked PyTorch.  "cats": the two-launch HIP path.
         "cats_rowmajor": flag_gemv_gemv_inner* (HF-layout down).  "cats_split": torch gate + HIP sparse up / down.
-        "cats_fused": "cats" with the post-attention norm and the residual add inside the two MLP launches."""
+        "cats_fused": "cats" with the post-attention norm and the residual add inside the two MLP launches.
+        "cats_fused_next": "cats_fused" whose launches also write the next layer's input norm (the final norm after the
+        last layer), so a decode step runs no stand-alone norm after the first layer's."""
         for layer in self.layers:
             m = layer.mlp
-            layer.fuse_norm_residual = mode == "cats_fused"
-            if mode == "cats_fused":
+            layer.fuse_norm_residual = mode in ("cats_fused", "cats_fused_next")
+            layer.fuse_next_norm = mode == "cats_fused_next"
+            if layer.fuse_norm_residual:
                 m.prepare_decode(3)
                 continue
             if mode == "dense":
@@ -267,7 +280,7 @@ class LlamaDecoder(nn.Module):
         return torch.stack(out)
 
 
-def compare_modes(model, prompt, n_tokens=32, modes=("cats_torch", "cats", "cats_fused")):
+def compare_modes(model, prompt, n_tokens=32, modes=("cats_torch", "cats", "cats_fused", "cats_fused_next")):
     """Agreement of the MLP modes on one model: the first mode decodes n_tokens greedily (eager); every mode is then
     run over that same token sequence and its per-step predictions are compared with the first mode's.
     Returns {mode: {"argmax_agreement": fraction of the n_tokens + 1 steps with the same top token,
@@ -376,7 +389,7 @@ def bench_decode(prompt_len=128, gen_len=256, sparsity=0.5, num_layers=32, seed=
     res = {"layers": cfg.num_layers, "prompt_len": prompt_len, "gen_len": gen_len, "target_sparsity": sparsity,
            "launch": "hipgraph" if use_graph else "stream", "setup_s": None}
     toks = {}
-    for mode in ("dense", "cats", "cats_fused"):
+    for mode in ("dense", "cats", "cats_fused", "cats_fused_next"):
         model.set_mlp_mode(mode)
         model.generate_greedy(prompt, min(gen_len, 8), use_graph=False)          # warm-up (workspaces, kernels)
         out, secs = model.generate_greedy(prompt, gen_len, use_graph=use_graph)
@@ -385,6 +398,7 @@ def bench_decode(prompt_len=128, gen_len=256, sparsity=0.5, num_layers=32, seed=
         res[f"{mode}_ms_per_token"] = round(secs / (gen_len - 1) * 1e3, 4)
     res["speedup"] = round(res["cats_tok_s"] / res["dense_tok_s"], 3)
     res["speedup_fused"] = round(res["cats_fused_tok_s"] / res["dense_tok_s"], 3)
+    res["speedup_fused_next"] = round(res["cats_fused_next_tok_s"] / res["dense_tok_s"], 3)
     res["mean_threshold"] = round(sum(thresholds) / len(thresholds), 5)
     # correctness of what was just timed, untimed: the kernel modes against the dense-masked PyTorch MLP (the reference's
     # sp_method 0) over the same 32 greedy tokens, and the sparsity the kernels actually met while decoding them
@@ -393,7 +407,7 @@ def bench_decode(prompt_len=128, gen_len=256, sparsity=0.5, num_layers=32, seed=
     res["layerwise_parity"] = layerwise_parity(model, prompt, 8)
     res["token_agreement"] = {"tokens": n_cmp + 1, "reference_mode": "cats_torch (dense-masked PyTorch MLP, sp_method 0)", **agree,
                               "free_running_common_prefix": {m: int((torch.cumprod((toks[m][:n_cmp] == toks["cats"][:n_cmp]).long(), 0)).sum())
-                                                             for m in ("cats_fused",)}}
+                                                             for m in ("cats_fused", "cats_fused_next")}}
     res["achieved_sparsity"] = {"mean": round(sum(sparsity) / len(sparsity), 4), "min": round(min(sparsity), 4), "max": round(max(sparsity), 4),
                                 "per_layer": [round(v, 4) for v in sparsity],
                                 "definition": "1 - neurons fetched / I per MLP call, averaged over the compared decode steps (batch 1: union = row sparsity)"}

@@ -143,6 +143,18 @@ class CatsMLP(nn.Module):
         return flash_gemv.cats_mlp_norm_residual(h, norm_weight, float(eps), self.gate_proj.weight, self.up_proj.weight,
                                                  self.wdown_t, float(self.dead_threshold))
 
+    def forward_norm_residual_norm(self, h, norm_weight, eps, next_norm_weight, next_eps):
+        """``(out, next)``: ``out`` as forward_norm_residual, ``next = next_norm_weight * rms_norm(out, next_eps)`` -- the
+        norm the following layer (or the model's final norm) would start with, written by the same two launches."""
+        if not (self.is_profile and self.sp_method == 3 and h.shape[1] == 1):
+            raise RuntimeError("CatsMLP.forward_norm_residual_norm: decode path only (prepare_decode(3), one token per row)")
+        if self.wdown_t is None:
+            raise RuntimeError("CatsMLP: sp_method 3 needs wdown_t (call prepare_decode() once after loading weights)")
+        import flash_gemv
+
+        return flash_gemv.cats_mlp_norm_residual_norm(h, norm_weight, float(eps), self.gate_proj.weight, self.up_proj.weight,
+                                                      self.wdown_t, float(self.dead_threshold), next_norm_weight, float(next_eps))
+
     def _dense_masked(self, x):
         post_act = self.act_fn(self.gate_proj(x))
         dead_neurons = post_act.abs() <= self.dead_threshold

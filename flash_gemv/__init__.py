@@ -99,6 +99,12 @@ def cats_mlp_norm_residual(h, norm_weight, eps, Wgate, Wup, Wdownt, threshold):
     return torch.ops.flash_gemv.cats_mlp_norm_residual(h, norm_weight, eps, Wgate, Wup, Wdownt, threshold)
 
 
+def cats_mlp_norm_residual_norm(h, norm_weight, eps, Wgate, Wup, Wdownt, threshold, next_norm_weight, next_eps):
+    """(out, next): out as cats_mlp_norm_residual, next = next_norm_weight * rms_norm(out, next_eps) from the same two
+    launches -- the input_layernorm of the following decoder layer (ugly_utils.py:1016-1057), or the final norm."""
+    return torch.ops.flash_gemv.cats_mlp_norm_residual_norm(h, norm_weight, eps, Wgate, Wup, Wdownt, threshold, next_norm_weight, next_eps)
+
+
 def cats_mlp_stats(x, Wgate, Wup, Wdownt, threshold):
     """cats_mlp that also returns the (B, I) bool flags and the number of neurons fetched (int32 tensor)."""
     return torch.ops.flash_gemv.cats_mlp_stats(x, Wgate, Wup, Wdownt, threshold)
@@ -130,4 +136,5 @@ __all__ = [
     "cats_mlp",
     "cats_mlp_stats",
     "cats_mlp_norm_residual",
+    "cats_mlp_norm_residual_norm",
 ]

@@ -247,6 +247,14 @@ def test_decode_loop_with_fused_layer_tail():
     assert torch.equal(fused, fused_g)
     agree = float((plain == fused).float().mean())
     assert agree >= 0.9, f"only {agree:.2f} of the greedy tokens agree between the fused and the unfused layer tail"
+    # the next layer's norm written by the MLP launches: the same arithmetic in another place, so the same tokens
+    # up to sums of squares added in another order
+    model.set_mlp_mode("cats_fused_next")
+    chained, _ = model.generate_greedy(prompt, 24, use_graph=False)
+    chained_g, _ = model.generate_greedy(prompt, 24, use_graph=True)
+    assert torch.equal(chained, chained_g)
+    agree = float((chained == fused).float().mean())
+    assert agree >= 0.9, f"only {agree:.2f} of the greedy tokens agree with and without the chained norm"
 
 
 def test_full_size_decoder_parity_agreement_and_sparsity():
@@ -276,7 +284,7 @@ def test_full_size_decoder_parity_agreement_and_sparsity():
     print(f"[full-size decode] {agree} mean sparsity {sum(sparsity) / len(sparsity):.4f}", flush=True)
     assert agree["self_consistent"]
     floor = agree["cats_torch_nudged"]
-    for mode in ("cats", "cats_fused"):
+    for mode in ("cats", "cats_fused", "cats_fused_next"):
         assert agree[mode]["argmax_agreement"] >= max(0.5, 1 - 2 * (1 - floor["argmax_agreement"])), (mode, agree)
         assert agree[mode]["max_logit_diff"] <= max(2 * floor["max_logit_diff"], 0.02 * floor["logit_scale"]), (mode, agree)
     assert len(sparsity) == 32 and all(0.45 <= v <= 0.55 for v in sparsity), sparsity
@@ -390,3 +398,25 @@ def test_bounded_soak_of_every_hot_entry_point_stays_bitwise_stable():
             torch.cuda.synchronize()
             assert torch.equal(gy1, want_g1) and torch.equal(gy8, want_g8), f"iteration {it}: graph replay differs from the eager result"
     assert calls == 240
+
+
+def test_probe_read_covers_the_whole_buffer():
+    """cats_probe_read writes nothing unless the fold of what one thread read equals its marker word: a buffer of zeros
+    with the marker planted at one position (first, last, odd offsets, inside the ragged tail of a span) must trip it,
+    a buffer without it must not.  So every 16-byte vector of the buffer is read by somebody."""
+    from cats_amd import capi
+
+    marker = 0x9E3779B9 - (1 << 32)  # as int32
+    n_words = (64 << 20) // 4 + 4 * 37  # 64 MiB and a ragged tail of 37 vectors
+    buf = torch.zeros(n_words, dtype=torch.int32, device="cuda")
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    capi.probe_read(buf, sink)
+    torch.cuda.synchronize()
+    assert int(sink.item()) == 0
+    for pos in (0, 5, n_words - 1, n_words // 2 + 3, n_words - 4 * 37 + 1, 4 * 511 + 2, 4 * 512 * 8 * 3 + 7):
+        buf[pos] = marker
+        sink.zero_()
+        capi.probe_read(buf, sink)
+        torch.cuda.synchronize()
+        assert int(sink.item()) == marker, f"word {pos} was not read"
+        buf[pos] = 0

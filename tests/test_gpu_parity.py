@@ -702,6 +702,54 @@ def test_norm_and_residual_folded_into_the_mlp(oracle, H, I, B, dtype):
     assert torch.equal(h2, got)
 
 
+@pytest.mark.parametrize("H,I,B,dtype", [(4096, 11008, 1, torch.float16), (4096, 1000, 2, torch.bfloat16), (512, 768, 4, torch.float16),
+                                         (1024, 640, 8, torch.bfloat16), (256, 333, 3, torch.float32), (2048, 512, 12, torch.float16)])
+def test_next_norm_written_by_the_finishing_launch(oracle, H, I, B, dtype):
+    """cats_mlp_norm_residual_norm: `out` carries the bits of cats_mlp_norm_residual (same launches), and `next` is the
+    RMS norm of exactly those stored values -- checked against the restated HF norm evaluated on the kernel's own `out`
+    (one fp32 sum of squares per row: the only difference is the order the squares are added in).  Twice on one
+    workspace (the arrival counter must be back at zero), then under a graph."""
+    m = make_mlp(H, I, B, dtype, seed=5 * H + I + B)
+    g = torch.Generator().manual_seed(H + I + 1)
+    h = (m["x"].float() * 1.7 - 0.2).to(dtype)
+    nw = (1.0 + 0.2 * torch.randn(H, generator=g)).to(dtype)
+    nw2 = (0.8 + 0.3 * torch.randn(H, generator=g)).to(dtype)
+    eps, eps2 = 1e-5, 1e-6
+    x_ref = oracle.torch_rms_norm(h, nw, eps)
+    t = float(torch.quantile(oracle.c_gate(x_ref, m["wg"], -1.0)[0].float().abs().flatten(), 0.5))
+    d = dev(dict(h=h, nw=nw, nw2=nw2, wg=m["wg"], wu=m["wu"], wdt=m["wdt"]))
+    ws = _ws(B, H, I)
+    want_out = capi.mlp_norm_residual(d["h"], d["nw"], eps, d["wg"], d["wu"], d["wdt"], t, ws)
+    tol = {torch.float16: dict(rtol=2e-3, atol=2e-3), torch.bfloat16: dict(rtol=1.6e-2, atol=1.6e-2), torch.float32: dict(rtol=1e-5, atol=1e-5)}[dtype]
+    for rep in range(2):
+        print(f"[case] next-norm dtype={dtype} B={B} H={H} I={I} rep={rep}", flush=True)
+        out, nxt = capi.mlp_norm_residual_norm(d["h"], d["nw"], eps, d["wg"], d["wu"], d["wdt"], t, d["nw2"], eps2, ws)
+        torch.cuda.synchronize()
+        assert torch.equal(out, want_out)
+        want_next = oracle.torch_rms_norm(out.cpu(), nw2, eps2)
+        torch.testing.assert_close(nxt.cpu().float(), want_next.float(), **tol)
+    # the whole chain against the oracle's restatement of the layer tail
+    ref = oracle.c_mlp(x_ref, m["wg"], m["wu"], m["wd"], t)
+    close(out.cpu(), h + ref["y"].to(dtype), dtype)
+    if B <= 8:
+        gr = torch.cuda.CUDAGraph()
+        hs = d["h"].clone()
+        with torch.cuda.graph(gr):
+            o_g, n_g = capi.mlp_norm_residual_norm(hs, d["nw"], eps, d["wg"], d["wu"], d["wdt"], t, d["nw2"], eps2, ws)
+        for rep in range(3):
+            capi.mlp(d["h"], d["wg"], d["wu"], d["wdt"], t, ws)   # eager work on the same workspace between replays
+            torch.cuda.synchronize()
+            gr.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(o_g, out) and torch.equal(n_g, nxt), f"replay {rep}"
+
+
+def test_next_norm_needs_rows_of_whole_reduction_blocks():
+    z = lambda *s: torch.zeros(*s, dtype=torch.float16, device="cuda")
+    with pytest.raises(capi.CatsError, match="shape"):
+        capi.mlp_norm_residual_norm(z(1, 72), z(72), 1e-5, z(64, 72), z(64, 72), z(64, 72), 0.1, z(72), 1e-5, _ws(1, 72, 64))
+
+
 def test_norm_residual_rejects_rows_that_do_not_fit_in_lds():
     H, I, B = 16384, 64, 8   # 8 x 32 KiB of fp16 activations
     z = lambda *s: torch.zeros(*s, dtype=torch.float16, device="cuda")
