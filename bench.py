@@ -96,6 +96,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run one 256 MiB device-to-device copy first: a kernel of known traffic for scaling rocprof counters")
     ap.add_argument("--print-csrc-hash", action="store_true", help="print the hash of the kernel sources (for a new counter record) and exit")
+    ap.add_argument("--contract", choices=("both", "y_out", "y_f32"), default="both",
+                    help="profiling aid: run the timed loops of one output contract only, so that a kernel trace or a counter run holds "
+                         "launches of one kind (y_f32: value is then the fp32-accumulate call and config.contract says so)")
     ap.add_argument("--path", type=int, default=0, help="1 = keep the call on the separate gate+up and sparse-down kernels")
     ap.add_argument("--gate-variant", type=int, default=0)
     ap.add_argument("--down-groups", type=int, default=0)
@@ -253,8 +256,9 @@ def main():
     # ---- headline: 50 % sparsity ---------------------------------------------------------------------------------
     t50 = thr[args.sparsity]
     k50 = active_count(t50)
-    us_eager = time_cats(t50, args.steps, args.warmup)
-    if args.no_graph:
+    only32 = args.contract == "y_f32"
+    us_eager = time_cats(t50, args.steps, args.warmup, f32=only32)
+    if args.no_graph or only32:
         us_graph, graph_steps = None, 0
     else:
         us_graph, graph_steps = time_cats_graph(t50, args.steps, args.warmup)
@@ -263,12 +267,18 @@ def main():
     # adds a microsecond to a 32 us kernel, over 400 it does not (the rocprofv3 trace of the same command agrees with
     # the long figure).  `value` itself is timed over exactly --steps calls.
     kernel_steps, kernel_warmup = max(args.steps, 400), max(args.warmup, 50)
-    us_k1 = time_cats(t50, kernel_steps, kernel_warmup, stage=1)
-    us_k2 = time_cats(t50, kernel_steps, kernel_warmup, stage=2)
-    rep_stats = per_rep_stats(t50, min(400, max(50, args.steps)))
+    if only32:  # one launch: the call is the kernel
+        us_k1, us_k2, rep_stats = us_eager, float("nan"), None
+    else:
+        us_k1 = time_cats(t50, kernel_steps, kernel_warmup, stage=1)
+        us_k2 = time_cats(t50, kernel_steps, kernel_warmup, stage=2)
+        rep_stats = per_rep_stats(t50, min(400, max(50, args.steps)))
     us_dense = time_dense(args.steps, args.warmup)
-    us_f32 = time_cats(t50, args.steps, args.warmup, f32=True)
-    us_f32_zero = time_cats(t50, args.steps, args.warmup, f32=True, zero_fill=True)
+    if args.contract == "y_out":
+        us_f32 = us_f32_zero = float("nan")
+    else:
+        us_f32 = us_eager if only32 else time_cats(t50, args.steps, args.warmup, f32=True)
+        us_f32_zero = time_cats(t50, args.steps, args.warmup, f32=True, zero_fill=True)
     # value is the plain stream-launch time of the call the decode path makes (fp16 y, two launches, bitwise
     # reproducible); the graph replay and the one-launch fp32-accumulate contract are reported beside it
     us, launch, steps_timed = us_eager, "stream", args.steps
@@ -293,7 +303,7 @@ def main():
         for s in SPARSITIES:
             k = active_count(thr[s])
             u = time_cats(thr[s], ssteps, swarm)
-            u32 = time_cats(thr[s], ssteps, swarm, f32=True)
+            u32 = time_cats(thr[s], ssteps, swarm, f32=True) if args.contract != "y_out" else float("nan")
             b = touched_bytes(sz, B, k)
             sweep.append(dict(target_sparsity=s, sparsity=round(1 - k / I, 4), us=round(u, 2), touched_MB=round(b / 1e6, 1),
                               GBps=round(b / u * 1e-3, 1), hbm_frac=round(b / u * 1e-3 / HBM_PEAK_GBPS, 4),
@@ -316,7 +326,7 @@ def main():
         "config": {"workload": "Llama-2-7B-shaped CATS MLP 4096->11008, fp16, batch 1, threshold at the 50th percentile of |SiLU(gate)|",
                    "hidden": H, "intermediate": I, "batch": B, "target_sparsity": args.sparsity,
                    "achieved_sparsity": round(1 - k50 / I, 4), "active_neurons": round(k50, 1), "weight_sets": args.sets,
-                   "launch": launch},
+                   "launch": launch, "contract": "y_f32 (fp32 accumulate, one launch)" if only32 else "y_out (fp16, two launches)"},
         "touched_bytes": int(tb),
         "achieved_GBps_touched": round(tb / us * 1e-3, 1),
         "hbm_frac_touched": round(tb / us * 1e-3 / HBM_PEAK_GBPS, 4),
@@ -387,7 +397,16 @@ def main():
             out["cpu_baseline"]["decode"] = decoder.cpu_decode_baseline(num_layers=4, gen_len=8, prompt_len=16, sparsity=0.5,
                                                                          threads=out["cpu_baseline"]["cores"])
 
-    print(json.dumps(out))
+    def no_nan(v):  # figures of a contract that was not run
+        if isinstance(v, float) and v != v:
+            return None
+        if isinstance(v, dict):
+            return {k: no_nan(w) for k, w in v.items()}
+        if isinstance(v, list):
+            return [no_nan(w) for w in v]
+        return v
+
+    print(json.dumps(no_nan(out)))
 
 
 def stream_ceiling(torch, capi, gib=1, reps=40):
@@ -485,7 +504,7 @@ def other_configs(torch, F, capi, L, steps, warmup, which):
     if "mistral" in which:
         run("mistral7b_bf16_heavy_tail", 4096, 14336, 1, torch.bfloat16, capi.BF16, [0.5, 0.7], heavy_tail=True)
     if "batch" in which:
-        for B in (2, 4, 8):
+        for B in (2, 4, 8, 16):
             run(f"llama7b_fp16_batch{B}_corr0.5", 4096, 11008, B, torch.float16, capi.F16, [0.5], corr=0.5)
     if "70b" in which:
         # the larger shape the reference smoke-tests (flash_gemv/test/test_fuse_gemv_cmp.py:662-676): 1.4 GB per weight set

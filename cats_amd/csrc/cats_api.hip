@@ -133,7 +133,7 @@ WsLayout ws_layout(int H, int I) {
   l.counters = o; o += kCounterBytes;
   l.partial = o;  o += align_up((size_t)kMaxGroups * B * ((size_t)(H + 511) / 512 * 512) * 4, 256);
   l.mask = o;     o += align_up((size_t)((I + 63) / 64) * 8, 256);
-  l.z32 = o;      o += align_up((size_t)B * I * 4, 256);
+  l.z32 = o;      o += align_up((size_t)CATS_MAX_BATCH * I * 4, 256);  // 16 rows: the one-pass gate + up of 9..16 rows fills it whole
   l.zt = o;       o += align_up((size_t)B * I * 4, 256);
   l.atmp = o;     o += align_up((size_t)B * I * 4, 256);
   l.fin = o;      o += align_up((size_t)B * H * 4, 256);  // finished columns as fp32, for the launch that also writes the next norm
@@ -651,6 +651,53 @@ static int mlp_pass(const void* x, const void* wgate, const void* wup, const voi
   return do_down(a.z32_out, true, wdown_t, acc, y_out, count_out, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
 }
 
+constexpr int kNotTaken = -1;  // mlp_wide: the call has to go the two-pass way
+
+// Whole MLP for 9..16 rows with W_gate and W_up read once: one matrix-core gate + up launch over all rows (two groups of
+// eight), then the sparse down pass per group of eight rows over the union mask of all rows.  Returns kNotTaken when the
+// type or the row length rules the one-pass kernel out (fp32, rows that are not 2048 or 4096 elements, the A/B knob).
+// norm_weight / residual / next: the layer-tail variants (x is then h); all optional.
+static int mlp_wide(const void* x, const void* norm_weight, float eps, const void* wgate, const void* wup, const void* wdown_t, void* y_out,
+                    float* y_f32, uint8_t* flag_out, int32_t* count_out, bool residual, const NextNorm& next, int B, int H, int I, int dtype,
+                    float threshold, void* ws, size_t ws_bytes, void* stream) {
+  if (B <= kKernelBatch || B > CATS_MAX_BATCH || dtype == CATS_F32) return kNotTaken;
+  int st = check_common(kKernelBatch, H, I, dtype);
+  if (st) return st;
+  if (!x || !wgate || !wup || !wdown_t || ((y_f32 == nullptr) == (y_out == nullptr))) return CATS_ERR_NULL;
+  if (!aligned16(x) || !aligned16(wgate) || !aligned16(wup) || !aligned16(wdown_t)) return CATS_ERR_ALIGN;
+  WsLayout l;
+  st = check_ws(ws, ws_bytes, H, I, l);
+  if (st) return st;
+  RowsArgs a;
+  fill_rows(a, x, wgate, H, I, B, dtype);
+  a.w2 = (const u32x4*)wup;
+  a.z32_out = (float*)((char*)ws + l.z32);
+  a.mask_out = (uint8_t*)ws + l.mask;
+  a.flag_out = flag_out;
+  a.t = round_through(dtype, threshold);
+  a.norm_w = (const u32x4*)norm_weight;
+  a.norm_eps = eps;
+  a.mma = g_tuning.gate_variant >= 0;
+#ifdef CATS_TIMING
+  a.tbuf = g_tbuf_rows;
+#endif
+  const bool ok = dtype == CATS_F16 ? rows_mma16_supported<F16>(a) : rows_mma16_supported<BF16>(a);
+  if (!ok) return kNotTaken;
+  const hipError_t e = dtype == CATS_F16 ? launch_rows_mma16<F16>(a, (hipStream_t)stream) : launch_rows_mma16<BF16>(a, (hipStream_t)stream);
+  if (e != hipSuccess) return CATS_ERR_LAUNCH;
+  const size_t sz = esz(dtype);
+  for (int b0 = 0; b0 < B; b0 += kKernelBatch) {
+    const int nb = B - b0 < kKernelBatch ? B - b0 : kKernelBatch;
+    NextNorm nx = next;
+    if (nx.out) nx.out = at_bytes(nx.out, (size_t)b0 * H * sz);
+    st = do_down(a.z32_out + (size_t)b0 * I, true, wdown_t, (float*)at_bytes((void*)y_f32, (size_t)b0 * H * 4), at_bytes(y_out, (size_t)b0 * H * sz),
+                 b0 == 0 ? count_out : nullptr, nb, H, I, dtype, (char*)ws, l, (hipStream_t)stream,
+                 residual ? at_cbytes(x, (size_t)b0 * H * sz) : nullptr, nullptr, nullptr, 0, nullptr, nx);
+    if (st) return st;
+  }
+  return CATS_OK;
+}
+
 static int up_down_pass(const void* x, const void* a_in, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,
                         int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
   int st = check_common(B, H, I, dtype);
@@ -788,6 +835,10 @@ int cats_mlp(const void* x, const void* wgate, const void* wup, const void* wdow
              uint8_t* flag_out, int32_t* count_out, int B, int H, int I, int dtype, float threshold, void* ws,
              size_t ws_bytes, void* stream) {
   const size_t sz = esz(dtype);
+  if (const int st = mlp_wide(x, nullptr, 0.f, wgate, wup, wdown_t, y_out, y_f32, flag_out, count_out, false, NextNorm(), B, H, I, dtype, threshold,
+                              ws, ws_bytes, stream);
+      st != kNotTaken)
+    return st;
   const bool union_count = count_out && B > kKernelBatch;  // a pass counts its own rows only: count the union of the flags instead
   if (union_count && !flag_out) {
     // no flags asked for: the passes write them into the workspace region of the row-major intermediate, which no MLP pass uses
@@ -916,6 +967,13 @@ int cats_mlp_norm_residual(const void* h, const void* norm_weight, float eps, co
                            const void* wdown_t, void* out, int B, int H, int I, int dtype, float threshold, void* ws,
                            size_t ws_bytes, void* stream) {
   const size_t sz = esz(dtype);
+  if (B > kKernelBatch && norm_weight && aligned16(norm_weight)) {
+    // in place (out == h) is fine here too: the gate + up launch has read all of h before the down passes write any row
+    if (const int st = mlp_wide(h, norm_weight, eps, wgate, wup, wdown_t, out, nullptr, nullptr, nullptr, true, NextNorm(), B, H, I, dtype,
+                                threshold, ws, ws_bytes, stream);
+        st != kNotTaken)
+      return st;
+  }
   return in_passes(B, [&](size_t b0, int nb) {
     return mlp_norm_residual_pass(at_cbytes(h, b0 * H * sz), norm_weight, eps, wgate, wup, wdown_t, at_bytes(out, b0 * H * sz), nb, H, I, dtype,
                                   threshold, ws, ws_bytes, stream);
@@ -929,6 +987,16 @@ int cats_mlp_norm_residual_norm(const void* h, const void* norm_weight, float ep
   if (!aligned16(next_norm_weight) || !aligned16(next_out)) return CATS_ERR_ALIGN;
   if (H % kReduceCols != 0) return CATS_ERR_SHAPE;
   const size_t sz = esz(dtype);
+  if (B > kKernelBatch && norm_weight && aligned16(norm_weight)) {
+    NextNorm next;
+    next.w = next_norm_weight;
+    next.eps = next_eps;
+    next.out = next_out;
+    if (const int st = mlp_wide(h, norm_weight, eps, wgate, wup, wdown_t, out, nullptr, nullptr, nullptr, true, next, B, H, I, dtype, threshold,
+                                ws, ws_bytes, stream);
+        st != kNotTaken)
+      return st;
+  }
   return in_passes(B, [&](size_t b0, int nb) {
     NextNorm next;
     next.w = next_norm_weight;

@@ -53,14 +53,24 @@ hipError_t launch_rows_one(const RowsArgs& a, hipStream_t stream) {
 // Matrix-core gate + up pass: one persistent workgroup per CU.
 template <class DT>
 struct MmaLaunch {
-  static bool supported(const RowsArgs&) { return false; }
+  static bool supported(const RowsArgs&, int = 1) { return false; }
   static hipError_t run(const RowsArgs&, bool, hipStream_t) { return hipErrorInvalidValue; }
+  static hipError_t run16(const RowsArgs&, hipStream_t) { return hipErrorInvalidValue; }
 };
 template <class DT>
 struct MmaLaunch16 {
-  static bool supported(const RowsArgs& a) {
+  static bool supported(const RowsArgs& a, int ng = 1) {
     const int steps = rows_mma_steps(a.K);
-    return (steps == 4 || steps == 8) && rows_mma_lds_bytes(a.K) <= 160 * 1024;
+    return (steps == 4 || steps == 8) && rows_mma_lds_bytes(a.K, ng) <= 160 * 1024;
+  }
+  // gate + up for 9..16 batch rows in one pass over the weights
+  static hipError_t run16(const RowsArgs& a, hipStream_t stream) {
+    const int cus = current_device_cus();
+    auto kern = rows_mma_steps(a.K) == 8 ? rows_mma_kernel<DT, 8, true, 2> : rows_mma_kernel<DT, 4, true, 2>;
+    const size_t lds = rows_mma_lds_bytes(a.K, 2);
+    if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
+    const int ntiles = (a.N + kMmaTileRows - 1) / kMmaTileRows;
+    return launch_kernel(kern, dim3(ntiles < cus ? ntiles : cus), dim3(kMmaThreads), lds, stream, a);
   }
   static hipError_t run(const RowsArgs& a, bool up, hipStream_t stream) {
     const int cus = current_device_cus();  // one workgroup per CU
@@ -158,6 +168,12 @@ hipError_t launch_fused<CATS_DT>(int bt, int grid, int stage, const FusedArgs& a
   }
   return hipSuccess;
 }
+
+template <>
+bool rows_mma16_supported<CATS_DT>(const RowsArgs& a) { return a.mma && MmaLaunch<CATS_DT>::supported(a, 2); }
+
+template <>
+hipError_t launch_rows_mma16<CATS_DT>(const RowsArgs& a, hipStream_t stream) { return MmaLaunch<CATS_DT>::run16(a, stream); }
 
 template <>
 hipError_t launch_rows<CATS_DT>(int mode, int bt, const RowsArgs& a, hipStream_t stream) {

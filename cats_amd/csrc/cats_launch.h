@@ -31,6 +31,13 @@ inline hipError_t launch_kernel(K kern, dim3 grid, dim3 block, size_t lds, hipSt
 template <class DT>
 hipError_t launch_rows(int mode, int bt, const RowsArgs& a, hipStream_t stream);
 
+// Gate + up for 9..16 batch rows in one pass over the weights (matrix-core kernel with two groups of eight rows):
+// whether the shape and type allow it, and the launch.
+template <class DT>
+bool rows_mma16_supported(const RowsArgs& a);
+template <class DT>
+hipError_t launch_rows_mma16(const RowsArgs& a, hipStream_t stream);
+
 template <class DT>
 hipError_t launch_down(int bt, bool zf32, const DownArgs& a, int block, hipStream_t stream);
 

@@ -49,16 +49,18 @@ constexpr int kMmaThreads = kMmaWaves * kWave;
 constexpr int kMmaTileRows = 8;
 constexpr int kMmaPart = 128;    // floats per wave in a partial buffer (the two useful quadrants)
 
-// dynamic LDS: x operands, gate partials, up partials
-inline size_t rows_mma_lds_bytes(int K) {
-  return (size_t)(K / 64) * kWave * sizeof(u32x4) + 2u * kMmaWaves * kMmaPart * sizeof(float);
+// dynamic LDS: x operands, gate partials, up partials -- each once per group of eight batch rows (ng = 1 or 2)
+inline size_t rows_mma_lds_bytes(int K, int ng = 1) {
+  return (size_t)ng * ((size_t)(K / 64) * kWave * sizeof(u32x4) + 2u * kMmaWaves * kMmaPart * sizeof(float));
 }
 // STEPS = 64-element k steps per wave per tile; the row length must be exactly kMmaWaves * STEPS * 64 so that no
 // load or MFMA sits behind a bounds check (control flow around loads in flight makes the compiler wait for them).
 inline int rows_mma_steps(int K) { return K % (kMmaWaves * 64) == 0 ? K / (kMmaWaves * 64) : 0; }
 
 // UP = false is the gate pass alone (activations, flags and union bits out; no up rows, no z).
-template <class DT, int STEPS, bool UP>
+// NG = 2 takes 9..16 batch rows in one pass over the weights: the second group of eight rows is a second x operand in
+// LDS and a second MFMA on the weight registers the first one just used, so the weights are still read once.
+template <class DT, int STEPS, bool UP, int NG = 1>
 __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
   typedef typename DT::st st;
   extern __shared__ u32x4 xs[];  // [nsteps][64] x operands, then the partial buffers
@@ -69,8 +71,10 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int kMmaSteps = STEPS;
   constexpr int nsteps = kMmaWaves * STEPS;
-  float* part_g = (float*)(xs + (size_t)nsteps * kWave);
-  float* part_u = part_g + kMmaWaves * kMmaPart;
+  constexpr int kXGroup = nsteps * kWave;             // operand vectors of one group of eight batch rows
+  constexpr int kPartGroup = kMmaWaves * kMmaPart;    // partial-sum floats of one group
+  float* part_g = (float*)(xs + (size_t)NG * kXGroup);
+  float* part_u = part_g + NG * kPartGroup;
 
   const int ntiles = (p.N + kMmaTileRows - 1) / kMmaTileRows;
   const int grid = gridDim.x;
@@ -100,13 +104,16 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
     for (int c = 0; c < kMmaSteps; c++) dst[c] = load_stream(src + c * stride);
   };
   auto multiply = [&](const u32x4 (&src)[kMmaSteps], float* part) {
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < kMmaSteps; c++) acc = Mma<DT>::run(src[c], xs[(s0 + c) * kWave + lane], acc);
-    if (keep) {
-      float* dst = part + wave * kMmaPart + slot;
+    for (int g = 0; g < NG; g++) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < 4; i++) dst[i * 32] = acc[i];
+      for (int c = 0; c < kMmaSteps; c++) acc = Mma<DT>::run(src[c], xs[g * kXGroup + (s0 + c) * kWave + lane], acc);
+      if (keep) {
+        float* dst = part + g * kPartGroup + wave * kMmaPart + slot;
+#pragma unroll
+        for (int i = 0; i < 4; i++) dst[i * 32] = acc[i];
+      }
     }
   };
   // wave 0, one thread per (row j of the tile, batch row b): adds the waves' partials in wave order
@@ -120,8 +127,13 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
   };
 
   // wave 0 carries the gate results of the previous tile until its up sums arrive
-  float prev_a = 0.f;
-  bool prev_act = false, prev_valid = false;
+  float prev_a[NG];
+  bool prev_act[NG], prev_valid[NG];
+#pragma unroll
+  for (int g = 0; g < NG; g++) {
+    prev_a[g] = 0.f;
+    prev_act[g] = prev_valid[g] = false;
+  }
   uint32_t prev_bits = 0u;
   int prev_row = 0;
 
@@ -129,25 +141,35 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
     multiply(gcur, part_g);
     issue(p.w, r + 2, gcur, false);
     __syncthreads();
-    float a = 0.f;
-    bool act = false, valid = false;
+    float a[NG];
+    bool act[NG], valid[NG];
+#pragma unroll
+    for (int g = 0; g < NG; g++) {
+      a[g] = 0.f;
+      act[g] = valid[g] = false;
+    }
     uint32_t bits8 = 0u;
     const int tile = blockIdx.x + r * grid;
     const int row = tile * kMmaTileRows + rj;
     if (wave == 0 && r < my_tiles) {
-      valid = row < p.N && rb < p.nb;
-      const float gr = DT::rnd(reduce(part_g));
-      a = DT::rnd(gr / (1.f + expf(-gr)));
-      act = valid && fabsf(a) > p.t;
-      const uint64_t bal = __ballot(act);
+      uint64_t bal = 0ull;
+#pragma unroll
+      for (int g = 0; g < NG; g++) {
+        const int b = g * 8 + rb;  // batch row of this thread in group g
+        valid[g] = row < p.N && b < p.nb;
+        const float gr = DT::rnd(reduce(part_g + g * kPartGroup));
+        a[g] = DT::rnd(gr / (1.f + expf(-gr)));
+        act[g] = valid[g] && fabsf(a[g]) > p.t;
+        bal |= __ballot(act[g]);
+        if (valid[g] && p.flag_out) p.flag_out[(size_t)b * p.N + row] = act[g] ? 1 : 0;
+        if (!UP && valid[g] && p.a_out) ((st*)p.a_out)[(size_t)b * p.N + row] = DT::fromf(a[g]);
+      }
 #pragma unroll
       for (int j = 0; j < 8; j++) bits8 |= ((bal >> (8 * j)) & 0xffull) ? (1u << j) : 0u;
       if (lane == 0) {
         s_any = bits8;
         if (p.mask_out) p.mask_out[tile] = (uint8_t)bits8;
       }
-      if (valid && p.flag_out) p.flag_out[(size_t)rb * p.N + row] = act ? 1 : 0;
-      if (!UP && valid && p.a_out) ((st*)p.a_out)[(size_t)rb * p.N + row] = DT::fromf(a);
     }
     __syncthreads();
     if (!UP) return;
@@ -155,14 +177,18 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
     multiply(uprev, part_u);
     __syncthreads();
     if (wave == 0) {
-      if (r >= 1 && prev_valid) {
-        const float u = reduce(part_u);
-        const float z = prev_act ? DT::rnd(prev_a * DT::rnd(u)) : 0.f;
-        const size_t o = (size_t)rb * p.N + prev_row;
-        if (p.z32_out && ((prev_bits >> rj) & 1u)) p.z32_out[o] = z;
-        if (p.zt_out) ((st*)p.zt_out)[o] = DT::fromf(z);
+#pragma unroll
+      for (int g = 0; g < NG; g++) {
+        if (r >= 1 && prev_valid[g]) {
+          const float u = reduce(part_u + g * kPartGroup);
+          const float z = prev_act[g] ? DT::rnd(prev_a[g] * DT::rnd(u)) : 0.f;
+          const size_t o = (size_t)(g * 8 + rb) * p.N + prev_row;
+          if (p.z32_out && ((prev_bits >> rj) & 1u)) p.z32_out[o] = z;
+          if (p.zt_out) ((st*)p.zt_out)[o] = DT::fromf(z);
+        }
+        prev_a[g] = a[g]; prev_act[g] = act[g]; prev_valid[g] = valid[g];
       }
-      prev_a = a; prev_act = act; prev_valid = valid; prev_bits = bits8; prev_row = row;
+      prev_bits = bits8; prev_row = row;
     }
   };
 
@@ -173,20 +199,24 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
   {
     // nsteps * 64 operand vectors over kMmaThreads threads = STEPS per thread, all loads in flight together;
     // batch rows past nb read row 0 and store zeros
-    u32x4 xv[STEPS];
+    u32x4 xv[NG][STEPS];
 #pragma unroll
-    for (int k = 0; k < STEPS; k++) {
-      const int i = tid + k * kMmaThreads;
-      const int step = i >> 6, l = i & 63;
-      const int n = l & 15, g = l >> 4, b = n & 7, kh = n >> 3;
-      xv[k] = p.x[(size_t)(b < p.nb ? b : 0) * p.row_vecs + step * 8 + kh * 4 + g];
-    }
+    for (int gb = 0; gb < NG; gb++)
 #pragma unroll
-    for (int k = 0; k < STEPS; k++) {
-      const int i = tid + k * kMmaThreads;
-      const int b = i & 7;
-      xs[i] = b < p.nb ? xv[k] : zero4();
-    }
+      for (int k = 0; k < STEPS; k++) {
+        const int i = tid + k * kMmaThreads;
+        const int step = i >> 6, l = i & 63;
+        const int n = l & 15, g = l >> 4, b = gb * 8 + (n & 7), kh = n >> 3;
+        xv[gb][k] = p.x[(size_t)(b < p.nb ? b : 0) * p.row_vecs + step * 8 + kh * 4 + g];
+      }
+#pragma unroll
+    for (int gb = 0; gb < NG; gb++)
+#pragma unroll
+      for (int k = 0; k < STEPS; k++) {
+        const int i = tid + k * kMmaThreads;
+        const int b = gb * 8 + (i & 7);
+        xs[gb * kXGroup + i] = b < p.nb ? xv[gb][k] : zero4();
+      }
     __builtin_amdgcn_sched_barrier(0);
     issue(p.w, 0, g0, false);
 #pragma unroll
@@ -199,21 +229,24 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
   if (p.norm_w) {
     // RMS norm in place.  Operand slot i = step * 64 + l holds batch row l % 8, vector step * 8 + (l % 16 / 8) * 4 + l / 16.
     // Wave b adds the squares of batch row b (kMmaWaves == 8 rows), in a fixed order.
-    __shared__ float s_scale[8];
-    {
+    __shared__ float s_scale[NG * 8];
+#pragma unroll
+    for (int gb = 0; gb < NG; gb++) {
       float ss = 0.f;
-      for (int q = lane; q < nsteps * 8; q += kWave) ss = vec_sumsq<DT>(xs[q * 8 + wave], ss);
+      for (int q = lane; q < nsteps * 8; q += kWave) ss = vec_sumsq<DT>(xs[gb * kXGroup + q * 8 + wave], ss);
       ss = wave_sum(ss);
-      if (lane == 0) s_scale[wave] = rsqrtf(ss / (float)p.K + p.norm_eps);
+      if (lane == 0) s_scale[gb * 8 + wave] = rsqrtf(ss / (float)p.K + p.norm_eps);
     }
     __syncthreads();
 #pragma unroll
-    for (int k = 0; k < STEPS; k++) {
-      const int i = tid + k * kMmaThreads;
-      const int step = i >> 6, l = i & 63;
-      const int n = l & 15, g = l >> 4, b = n & 7, kh = n >> 3;
-      if (b < p.nb) xs[i] = vec_norm_apply<DT>(xs[i], s_scale[b], p.norm_w[step * 8 + kh * 4 + g]);
-    }
+    for (int gb = 0; gb < NG; gb++)
+#pragma unroll
+      for (int k = 0; k < STEPS; k++) {
+        const int i = tid + k * kMmaThreads;
+        const int step = i >> 6, l = i & 63;
+        const int n = l & 15, g = l >> 4, b = gb * 8 + (n & 7), kh = n >> 3;
+        if (b < p.nb) xs[gb * kXGroup + i] = vec_norm_apply<DT>(xs[gb * kXGroup + i], s_scale[b], p.norm_w[step * 8 + kh * 4 + g]);
+      }
     __syncthreads();
   }
   CATS_RSTAMP(1);

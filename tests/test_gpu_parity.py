@@ -767,21 +767,46 @@ def test_llama70b_shape(oracle, B):
     check_mlp_case(oracle, m, t, tag=f"llama70b-fp16-B{B}")
 
 
-@pytest.mark.parametrize("H,I,B,dtype", [(4096, 1000, 16, torch.float16), (512, 333, 11, torch.bfloat16), (260, 96, 9, torch.float32)])
-def test_batches_of_nine_to_sixteen_rows_run_in_two_passes(oracle, H, I, B, dtype):
-    """The reference's kernels are instantiated up to 16 rows (fuse_gemv_cmp_cuda.cu:2368-2400); here such a batch is
-    two passes of at most 8 rows over the weights, row for row the same arithmetic."""
+@pytest.mark.parametrize("H,I,B,dtype", [(4096, 1000, 16, torch.float16), (512, 333, 11, torch.bfloat16), (260, 96, 9, torch.float32),
+                                         (2048, 1536, 9, torch.bfloat16), (4096, 11008, 12, torch.float16), (4096, 2048, 16, torch.bfloat16)])
+def test_batches_of_nine_to_sixteen_rows(oracle, H, I, B, dtype):
+    """The reference's kernels are instantiated up to 16 rows (fuse_gemv_cmp_cuda.cu:2368-2400).  Here 16-bit rows of 2048
+    or 4096 elements take one matrix-core gate + up pass over all rows (W_gate and W_up read once) and the down pass per
+    group of eight rows over the union mask; every other case is two passes of at most 8 rows.  Either way: the full
+    parity case, and rows 8.. of the big batch against the same rows run as a batch of their own (same flags, bit for
+    bit; outputs to the parity tolerance -- the union of sixteen rows orders the down sums differently)."""
     m = make_mlp(H, I, B, dtype, seed=B + H, corr=0.3)
     a_abs = oracle.c_gate(m["x"], m["wg"], -1.0)[0].float().abs().flatten()
-    check_mlp_case(oracle, m, float(torch.quantile(a_abs, 0.5)), tag=f"two-pass-B{B}")
-    # row b of the big batch equals row b of its own pass
+    t = float(torch.quantile(a_abs, 0.5))
+    check_mlp_case(oracle, m, t, tag=f"rows-9-to-16-B{B}")
     d = dev(m)
     ws = _ws(B, H, I)
-    t = float(torch.quantile(a_abs, 0.5))
-    y_all = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws)
-    y_hi = capi.mlp(d["x"][8:].contiguous(), d["wg"], d["wu"], d["wdt"], t, ws)
+    y_all, f_all, _ = capi.mlp(d["x"], d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
+    y_hi, f_hi, _ = capi.mlp(d["x"][8:].contiguous(), d["wg"], d["wu"], d["wdt"], t, ws, want_flag=True, want_count=True)
     torch.cuda.synchronize()
-    assert torch.equal(y_all[8:], y_hi)
+    if B - 8 >= 3 or dtype == torch.float32 or H not in (2048, 4096):   # same gate kernel in both calls: same activations
+        assert torch.equal(f_all[8:], f_hi)
+    close(y_all[8:].cpu(), y_hi.cpu(), dtype)
+    # the layer tail through the same path, in place and with the next norm
+    g = torch.Generator().manual_seed(B)
+    nw = (1.0 + 0.2 * torch.randn(H, generator=g)).to(dtype).cuda()
+    h = (d["x"].float() * 1.5).to(dtype)
+    want = capi.mlp_norm_residual(h[:8].contiguous(), nw, 1e-5, d["wg"], d["wu"], d["wdt"], t, ws)
+    want_hi = capi.mlp_norm_residual(h[8:].contiguous(), nw, 1e-5, d["wg"], d["wu"], d["wdt"], t, ws)
+    got = capi.mlp_norm_residual(h, nw, 1e-5, d["wg"], d["wu"], d["wdt"], t, ws)
+    torch.cuda.synchronize()
+    close(got[:8].cpu(), want.cpu(), dtype)
+    close(got[8:].cpu(), want_hi.cpu(), dtype)
+    if H % 32 == 0:
+        out, nxt = capi.mlp_norm_residual_norm(h, nw, 1e-5, d["wg"], d["wu"], d["wdt"], t, nw, 1e-6, ws)
+        torch.cuda.synchronize()
+        assert torch.equal(out, got)
+        ntol = {torch.float16: dict(rtol=2e-3, atol=2e-3), torch.bfloat16: dict(rtol=1.6e-2, atol=1.6e-2), torch.float32: dict(rtol=1e-5, atol=1e-5)}[dtype]
+        torch.testing.assert_close(nxt.cpu().float(), oracle.torch_rms_norm(out.cpu(), nw.cpu(), 1e-6).float(), **ntol)
+    h2 = h.clone()
+    capi.mlp_norm_residual(h2, nw, 1e-5, d["wg"], d["wu"], d["wdt"], t, ws, out=h2)
+    torch.cuda.synchronize()
+    assert torch.equal(h2, got)
 
 
 def test_batch_above_sixteen_is_an_error_not_a_crash():
