@@ -299,8 +299,12 @@ def compare_modes(model, prompt, n_tokens=32, modes=("cats_torch", "cats", "cats
     sparsity = None
 
     def score(lg):
+        # per-step distance from the reference run: rounding-level differences start small and grow as flipped mask bits
+        # accumulate in the KV cache; a defect in one layer's arithmetic would be large from the first step on
+        by_step = (lg - ref).abs().amax(-1)
         return {"argmax_agreement": round(float((lg.argmax(-1) == ref.argmax(-1)).float().mean()), 4),
-                "max_logit_diff": round(float((lg - ref).abs().max()), 5), "logit_scale": round(float(ref.abs().max()), 4)}
+                "max_logit_diff": round(float((lg - ref).abs().max()), 5), "logit_scale": round(float(ref.abs().max()), 4),
+                "max_logit_diff_by_step": [round(float(v), 4) for v in by_step[:: max(1, by_step.numel() // 8)]]}
 
     for mode in modes:
         model.set_mlp_mode(mode)

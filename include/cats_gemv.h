@@ -57,7 +57,9 @@ typedef enum {
   CATS_ERR_SCRATCH = 8     /* cats_mlp_noalloc: the call does not fit the library's built-in scratch */
 } cats_status_t;
 
-#define CATS_MAX_BATCH 16  /* 1..8 rows are one pass over the weights; 9..16 rows are two (the weights are read per pass) */
+#define CATS_MAX_BATCH 16  /* 1..8 rows are one pass over the weights.  9..16 rows: the whole-MLP entry points read W_gate and W_up
+                            * once (16-bit types, rows of 2048 or 4096 elements) and run the sparse down pass per group of eight
+                            * rows; every other case is two passes of at most eight rows */
 
 /* Library identification / error text.  No reference counterpart (the reference printf()s and exit()s:
  * flash_gemv/csrc/cuda/fuse_gemv_cmp_cuda.cu:25-33,2397-2400). */
@@ -135,13 +137,17 @@ int cats_down_index(const void* z, const void* wdown_t, const int64_t* idx, int 
 int cats_gate_up(const void* x, const void* wgate, const void* wup, void* out, uint8_t* flag_out,
                  int B, int H, int I, int dtype, float threshold, void* stream);
 
-/* Whole CATS MLP with neuron-major down weights, two launches.  1..2 rows: one streaming kernel in which every workgroup
- * takes its neurons through gate, up and down and leaves (B,H) partial sums, then a reduction over the workgroups;
- * more rows (and y_f32 mode): gate+up kernel, then sparse down kernel.
- *   y_out != NULL : (B,H) in dtype;  y_f32 != NULL : fp32 accumulate into the caller's pre-zeroed (B,H).
+/* Whole CATS MLP with neuron-major down weights.  1..2 rows: one streaming kernel in which every workgroup takes its
+ * neurons through gate, up and down; more rows: gate+up kernel, then sparse down kernel.
+ *   y_out != NULL : (B,H) in dtype.  The workgroups leave fp32 partial sums and a second launch adds them in a fixed
+ *                   order: the result is bitwise reproducible from run to run.
+ *   y_f32 != NULL : fp32 accumulate into the caller's (B,H), which the caller has zeroed (or which holds what the result
+ *                   is to be added to) -- the contract of the reference ops named below.  At 1..2 rows this is ONE launch:
+ *                   the streaming kernel adds its sums into y_f32 with fp32 atomics (the order, and so the last bits,
+ *                   vary from run to run).
  * flag_out (B,I) optional.  count_out (device int32, optional) receives the number of neurons active in any row of the
- * batch (for up to 8 rows that is the number of neurons fetched; 9..16 rows fetch per pass and one small kernel counts
- * the union of the flags afterwards).
+ * batch (the number of neurons fetched; where 9..16 rows run as two passes one small kernel counts the union of the
+ * flags afterwards).  With y_f32 and count_out at 1..2 rows a second, tiny launch totals the count.
  * Replaces flag_gemv_gemv_atomic, fuse_gemv_gemv_gemv, fuse_gemv_flag_gemv_gemv (flash_gemv.py:12-16,30-31;
  * fuse_gemv_cmp_cuda.cu:786-1244,2196-2253) and the composite gemv_gemv_triton / flag_gemv_gemv_triton
  * (flash_gemv/flash_gemv/__init__.py:38-48). */

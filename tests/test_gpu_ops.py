@@ -284,9 +284,11 @@ def test_full_size_decoder_parity_agreement_and_sparsity():
     print(f"[full-size decode] {agree} mean sparsity {sum(sparsity) / len(sparsity):.4f}", flush=True)
     assert agree["self_consistent"]
     floor = agree["cats_torch_nudged"]
+    note = ("token agreement of a random-init 32-layer decoder only bounds gross errors (the control moves as much from a 0.1 % "
+            "threshold nudge); the parity gate of this test is the layerwise check above")
     for mode in ("cats", "cats_fused", "cats_fused_next"):
-        assert agree[mode]["argmax_agreement"] >= max(0.5, 1 - 2 * (1 - floor["argmax_agreement"])), (mode, agree)
-        assert agree[mode]["max_logit_diff"] <= max(2 * floor["max_logit_diff"], 0.02 * floor["logit_scale"]), (mode, agree)
+        assert agree[mode]["argmax_agreement"] >= max(0.5, 1 - 2 * (1 - floor["argmax_agreement"])), (note, mode, agree)
+        assert agree[mode]["max_logit_diff"] <= max(2 * floor["max_logit_diff"], 0.02 * floor["logit_scale"]), (note, mode, agree)
     assert len(sparsity) == 32 and all(0.45 <= v <= 0.55 for v in sparsity), sparsity
     del model
     torch.cuda.empty_cache()
