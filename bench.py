@@ -89,6 +89,7 @@ def main():
     ap.add_argument("--extra", default="mistral,batch,70b,entry",
                     help="which of the other measurements to run: mistral (bf16, heavy-tailed), batch (2/4/8), 70b (8192->28672), "
                          "entry (each drop-in entry point alone)")
+    ap.add_argument("--batches", default="2,4,8,16", help="with --extra batch: the batch sizes to run")
     ap.add_argument("--entries", default="", help="with --extra entry: comma-separated entry points to time (default: all)")
     ap.add_argument("--no-graph", action="store_true", help="time plain stream launches only")
     ap.add_argument("--decode", action="store_true", help="(default) run the 32-layer decode loop (config 5)")
@@ -376,7 +377,8 @@ def main():
     if extra & {"mistral", "batch", "70b"}:
         del sets
         torch.cuda.empty_cache()
-        out["other_configs"] = other_configs(torch, F, capi, L, max(200, args.steps // 4), max(50, args.warmup // 4), extra)
+        out["other_configs"] = other_configs(torch, F, capi, L, max(200, args.steps // 4), max(50, args.warmup // 4), extra,
+                                             [int(b) for b in args.batches.split(",") if b.strip()], args.contract)
 
     if "entry" in extra:
         out["entry_points"] = entry_points(torch, F, capi, max(200, args.steps // 4), max(50, args.warmup // 4),
@@ -432,7 +434,7 @@ def stream_ceiling(torch, capi, gib=1, reps=40):
             "us_per_pass": round(us, 2), "kernel": "read_probe_kernel (cats_probe_read): read-only, nothing written"}
 
 
-def other_configs(torch, F, capi, L, steps, warmup, which):
+def other_configs(torch, F, capi, L, steps, warmup, which, batches=(2, 4, 8, 16), contract="both"):
     """The remaining single-layer configurations: Mistral-7B shape in bf16 with heavy-tailed gate rows (50 / 70 %), and
     the Llama fp16 layer at batch 2 / 4 / 8 with pairwise-correlated rows (per-row masks, union gathering), and the
     Llama-70B-shaped layer at batch 1."""
@@ -489,10 +491,10 @@ def other_configs(torch, F, capi, L, steps, warmup, which):
             k = sum(ks) / len(ks)
             prepared = [(p(x), p(st["wg"]), p(st["wu"]), p(st["wdt"]), p(y), None, None, None, B, Hh, Ii, code, ctypes.c_float(t), p(ws.buf), ws.nbytes, stream)
                         for st in sets]
-            us = timed(lambda i: L.cats_mlp(*prepared[i % nsets]))
+            us = timed(lambda i: L.cats_mlp(*prepared[i % nsets])) if contract != "y_f32" else float("nan")
             # the fp32-accumulate contract (adds into the caller's fp32 buffer; one launch at 1..2 rows)
             prepared32 = [a[:4] + (None, p(y32)) + a[6:] for a in prepared]
-            us32 = timed(lambda i: L.cats_mlp(*prepared32[i % nsets]))
+            us32 = timed(lambda i: L.cats_mlp(*prepared32[i % nsets])) if contract != "y_out" else float("nan")
             tb = sz * Hh * Ii + 2 * sz * Hh * k + sz * B * (2 * Hh + Ii) + 4 * k + 4
             res.append(dict(config=name, batch=B, row_sparsity_target=s, union_sparsity=round(1 - k / Ii, 4), us=round(us, 2),
                             touched_MB=round(tb / 1e6, 1), GBps=round(tb / us * 1e-3, 1), hbm_frac=round(tb / us * 1e-3 / HBM_PEAK_GBPS, 4),
@@ -504,7 +506,7 @@ def other_configs(torch, F, capi, L, steps, warmup, which):
     if "mistral" in which:
         run("mistral7b_bf16_heavy_tail", 4096, 14336, 1, torch.bfloat16, capi.BF16, [0.5, 0.7], heavy_tail=True)
     if "batch" in which:
-        for B in (2, 4, 8, 16):
+        for B in batches:
             run(f"llama7b_fp16_batch{B}_corr0.5", 4096, 11008, B, torch.float16, capi.F16, [0.5], corr=0.5)
     if "70b" in which:
         # the larger shape the reference smoke-tests (flash_gemv/test/test_fuse_gemv_cmp.py:662-676): 1.4 GB per weight set

@@ -546,9 +546,6 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       float z[B];
 #pragma unroll
       for (int b = 0; b < B; b++) z[b] = 0.f;
-#ifdef CATS_TIMING
-      if (p.tbuf && lane == 0) atomicMax((unsigned long long*)&p.tbuf[(size_t)blockIdx.x * 8 + 7], (unsigned long long)wall_clock64());
-#endif
       if (any) {  // wave-uniform
         // the down waves may send for this neuron's W_down^T row now: it travels while the W_up row does
         if (lane == 0) __hip_atomic_store(&sl.state[curslot], kSlotAnnounced, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -679,7 +676,6 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       nlive += ba.cnt;
       break;
     }
-    CATS_FSTAMP(lane == 0 && d == 0 && bb.cnt > 0, 5);
     fused_down_issue<B, KV, RB>(bb, p.wd, p.row_vecs, p.x, vidx);
     fused_resolve<B, KV, RB, ANN>(ba, sl);
     fused_down_consume<DT, B, KV, RB>(ba, acc);
@@ -692,7 +688,6 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       nlive += bb.cnt;
       break;
     }
-    CATS_FSTAMP(lane == 0 && d == 0 && ba.cnt > 0, 5);
     fused_down_issue<B, KV, RB>(ba, p.wd, p.row_vecs, p.x, vidx);
     fused_resolve<B, KV, RB, ANN>(bb, sl);
     fused_down_consume<DT, B, KV, RB>(bb, acc);
