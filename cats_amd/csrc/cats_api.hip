@@ -275,8 +275,13 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   d.flags = flags;
   d.idx = idx;
   d.M = M;
+  // The caller's fp32 accumulator: up to two rows the workgroups add into it themselves (one launch); from three rows
+  // on that is eight or more rows of atomics per workgroup and slower than leaving partial sums for the reduction launch,
+  // which then adds the total into the accumulator (measured at 4 / 8 / 16 rows: 53.9 / 64.6 / 104 us against 52.8 / 59.1 / 87.5).
+  const bool reduce_into_y32 = y32 != nullptr && y_out == nullptr && B >= 3;
   d.y32 = y32;
   d.y_out = y_out;
+  d.partial_out = (y_out != nullptr || reduce_into_y32) ? 1 : 0;
   d.partial = (float*)(ws + l.partial);
   d.count_out = count_out;
   d.H = H; d.I = I; d.nb = B;
@@ -304,12 +309,13 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   else if (dtype == CATS_BF16) e = launch_down<BF16>(bt, zf32, d, block, s);
   else e = launch_down<F32>(bt, zf32, d, block, s);
   if (e != hipSuccess) return CATS_ERR_LAUNCH;
-  if (y_out == nullptr) return CATS_OK;
-  // y_out mode: the groups' partial sums are added, rounded (and the residual added) by the reduction launch
+  if (!d.partial_out) return CATS_OK;
+  // the groups' partial sums are added by the reduction launch: rounded into y_out (and the residual added), or added to y32
   ReduceArgs r;
   memset(&r, 0, sizeof(r));
   r.partial = d.partial;
   r.y_out = y_out;
+  r.y32_acc = reduce_into_y32 ? y32 : nullptr;
   r.residual = residual;
   r.bias = bias;
   r.H = H;

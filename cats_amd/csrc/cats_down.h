@@ -10,7 +10,9 @@
 //     No atomics on data (32 workgroups adding into the same 16 cache lines serialise for microseconds), a fixed
 //     summation order (bitwise reproducible output), nothing to zero between calls, no synchronisation between
 //     workgroups other than the launch boundary.
-//   * y32 (caller's fp32 accumulator, "atomic_gemv" semantics): one fp32 atomic per column per workgroup.
+//   * y32 (caller's fp32 accumulator, "atomic_gemv" semantics): one fp32 atomic per column per workgroup -- up to two
+//     batch rows, where saving the second launch is worth it; from three rows on the partial sums go the first way and
+//     the reduction launch adds their total into the accumulator.
 // blockIdx % nslab picks the slab, so with 8 slabs every XCD (workgroups are dealt round-robin over the 8
 // XCDs) streams one slab.
 //
@@ -31,9 +33,10 @@ struct DownArgs {
   const uint8_t* flags;   // alternative to mask: (nb, I) flag bytes, OR-ed over the batch on the fly; NULL = use mask
   const int64_t* idx;     // alternative to both: an index list of M weight rows (any order, duplicates add up, entries outside
   int M;                  //   [0, I) contribute nothing); z is then (nb, M), aligned with the list, and the groups split the list
-  float* y32;             // (nb, H) the caller's fp32 accumulator (atomics), used when y_out == NULL
+  float* y32;             // (nb, H) the caller's fp32 accumulator, added to with atomics when partial_out is not set
   void* y_out;            // (nb, H) dtype
-  float* partial;         // y_out mode: [ngroup][nb][H] fp32 partial sums, finished by reduce_partials_kernel
+  int partial_out;        // the folded sums go to `partial` and reduce_partials_kernel finishes (into y_out, or adds into y32)
+  float* partial;         // [ngroup][nb][H] fp32 partial sums
   int32_t* count_out;     // optional: number of active neurons
   int H, I, nb;
   int row_vecs;           // H / VEC
@@ -275,7 +278,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
       }
       const int col = (slab * kWave + l) * VEC + 4 * h;
       if (col < p.H) {  // H is a multiple of VEC, so a quad is inside or outside as a whole
-        if (p.y_out) {
+        if (p.partial_out) {
           *(float4*)&p.partial[((size_t)group * p.nb + b0 + b) * p.H + col] = s4;
         } else if (n > 0) {
           float* y = &p.y32[(size_t)(b0 + b) * p.H + col];

@@ -99,6 +99,7 @@ struct ReduceArgs {
   const float* partial;  // [G][BH]
   const int32_t* counts; // [G]
   void* y_out;           // (nb, H) dtype, flattened to BH
+  float* y32_acc;        // instead of y_out: (nb, H) fp32 that the sums are added to, unrounded (the fp32-accumulate contract)
   const void* residual;  // optional (nb, H) dtype; may alias y_out
   const void* bias;      // optional (H,) dtype, added in fp32 before the rounding
   int H;                 // row length of y (for the bias)
@@ -579,7 +580,7 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
       }
       cur = nxt;
       curslot = nxtslot;
-      // what the ticket taken at the top of this round is worth
+      // what the ticket taken at the top of this pass of the loop is worth
       nxt = -1;
       nxtslot = pend;
       if (pend >= 0) {  // wave-uniform
@@ -800,8 +801,12 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(ReduceArgs p) {
 #pragma unroll
       for (int l = 0; l < kReduceLanes; l++) tot += s_sum[l][tid];
       if (p.bias) tot += DT::tof(((const st*)p.bias)[c % p.H]);
-      if (p.residual) tot = DT::rnd(tot) + DT::tof(((const st*)p.residual)[c]);
-      ((st*)p.y_out)[c] = DT::fromf(tot);
+      if (p.y32_acc) {
+        p.y32_acc[c] += tot;  // one thread per column, nobody else touches it during the call
+      } else {
+        if (p.residual) tot = DT::rnd(tot) + DT::tof(((const st*)p.residual)[c]);
+        ((st*)p.y_out)[c] = DT::fromf(tot);
+      }
     }
   }
   if (p.norm2_out) {

@@ -110,3 +110,26 @@ def test_torch_ops_reject_cpu_tensors():
     out, flag = torch.zeros(1, 1, 96, dtype=torch.float16), torch.zeros(96, dtype=torch.bool)
     with pytest.raises(RuntimeError, match="GPU"):
         flash_gemv.fuse_gemv_flag_local(x, w, out, flag, 0.1)
+
+
+def test_argument_validation_of_the_newer_entry_points():
+    """cats_mlp_norm_residual_norm and cats_probe_read reject bad arguments before any HIP call."""
+    from cats_amd import capi
+
+    L = capi.lib()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 255) // 256 * 256)
+    odd = ctypes.c_void_p(p.value + 4)
+    big = 1 << 30
+    nrn = L.cats_mlp_norm_residual_norm
+    assert nrn(p, p, 1e-5, p, p, p, p, None, 1e-5, p, 1, 64, 96, 0, 0.1, p, big, None) == 5      # next norm weight missing
+    assert nrn(p, p, 1e-5, p, p, p, p, p, 1e-5, None, 1, 64, 96, 0, 0.1, p, big, None) == 5      # next output missing
+    assert nrn(p, p, 1e-5, p, p, p, p, odd, 1e-5, p, 1, 64, 96, 0, 0.1, p, big, None) == 3       # misaligned weight
+    assert nrn(p, p, 1e-5, p, p, p, p, p, 1e-5, p, 1, 72, 96, 0, 0.1, p, big, None) == 2         # H % 32 != 0
+    assert nrn(p, p, 1e-5, p, p, p, p, p, 1e-5, p, 17, 64, 96, 0, 0.1, p, big, None) == 4        # batch
+    probe = L.cats_probe_read
+    probe.argtypes, probe.restype = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_void_p], ctypes.c_int
+    assert probe(None, 64, p, None) == 5
+    assert probe(p, 0, p, None) == 3
+    assert probe(p, 24, p, None) == 3
+    assert probe(odd, 64, p, None) == 3
