@@ -284,7 +284,7 @@ def main():
     # reproducible); the graph replay and the one-launch fp32-accumulate contract are reported beside it
     us, launch, steps_timed = us_eager, "stream", args.steps
     tb = touched_bytes(sz, B, k50)
-    ceiling = stream_ceiling(torch, capi)
+    ceiling = stream_ceiling(torch, capi, tb)
     single_pass = args.path != 1
     partial_bytes = 0
     if single_pass:
@@ -342,9 +342,12 @@ def main():
             "hbm_frac_touched": round(tb / us_f32 * 1e-3 / HBM_PEAK_GBPS, 4),
             "us_with_zero_fill": round(us_f32_zero, 3),
             "hbm_frac_touched_with_zero_fill": round(tb / us_f32_zero * 1e-3 / HBM_PEAK_GBPS, 4),
+            "plain_read_time_over_call_time": round(ceiling["same_bytes_as_one_call"]["us"] / us_f32, 4),
         },
         "stream_ceiling": ceiling,
         "frac_of_stream_ceiling": round(tb / us * 1e-3 / ceiling["GBps"], 4),
+        "plain_read_of_the_same_bytes_us": ceiling["same_bytes_as_one_call"]["us"],
+        "plain_read_time_over_call_time": round(ceiling["same_bytes_as_one_call"]["us"] / us, 4),
         "dense_fp16_us": round(us_dense, 3),
         "dense_GBps": round(3 * sz * H * I / us_dense * 1e-3, 1),
         "speedup_vs_dense": round(us_dense / us, 3),
@@ -411,27 +414,39 @@ def main():
     print(json.dumps(no_nan(out)))
 
 
-def stream_ceiling(torch, capi, gib=1, reps=40):
+def stream_ceiling(torch, capi, call_bytes, gib=1, reps=40):
     """Read-stream bandwidth this GPU reaches: cats_probe_read (read-only, the same 128-bit streaming loads as the weight
-    rows) over a 1 GiB buffer, four times the 256 MB memory-side cache, timed with events on the launch stream."""
+    rows) over a 1 GiB buffer, four times the 256 MB memory-side cache, timed with events on the launch stream.  And the
+    same kernel over exactly the bytes one headline call touches (slices of the buffer in turn, so nothing is cached):
+    the time a perfectly balanced, dependency-free read of those bytes takes as one launch -- a launch's fixed cost
+    weighs more on 181 MB than on 1 GiB."""
     buf = torch.empty(gib << 30, dtype=torch.uint8, device="cuda")
     buf.fill_(1)
     sink = torch.zeros(1, dtype=torch.int32, device="cuda")
-    for _ in range(5):
-        capi.probe_read(buf, sink)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        capi.probe_read(buf, sink)
-    e1.record()
-    torch.cuda.synchronize()
-    us = e0.elapsed_time(e1) * 1e3 / reps
+
+    def timed(fn, n):
+        for i in range(5):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(n):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / n
+
+    us = timed(lambda i: capi.probe_read(buf, sink), reps)
     nbytes = buf.numel()
-    del buf
+    nb = int(call_bytes) // 16 * 16
+    slices = [buf[i * nb:(i + 1) * nb] for i in range(nbytes // nb)]
+    us_call = timed(lambda i: capi.probe_read(slices[i % len(slices)], sink), 10 * reps)
+    del buf, slices
     torch.cuda.empty_cache()
     return {"GBps": round(nbytes / us * 1e-3, 1), "frac_of_peak": round(nbytes / us * 1e-3 / HBM_PEAK_GBPS, 4), "bytes": nbytes,
-            "us_per_pass": round(us, 2), "kernel": "read_probe_kernel (cats_probe_read): read-only, nothing written"}
+            "us_per_pass": round(us, 2), "kernel": "read_probe_kernel (cats_probe_read): read-only, nothing written",
+            "same_bytes_as_one_call": {"bytes": nb, "us": round(us_call, 2), "GBps": round(nb / us_call * 1e-3, 1),
+                                       "frac_of_peak": round(nb / us_call * 1e-3 / HBM_PEAK_GBPS, 4)}}
 
 
 def other_configs(torch, F, capi, L, steps, warmup, which, batches=(2, 4, 8, 16), contract="both"):

@@ -81,17 +81,20 @@ __global__ __launch_bounds__(512) void read_probe_kernel(const u32x4* __restrict
   const size_t lo = (size_t)blockIdx.x * span < n16 ? (size_t)blockIdx.x * span : n16;
   const size_t hi = lo + span < n16 ? lo + span : n16;
   uint32_t acc = 0;
-  size_t i = lo + threadIdx.x;
-  for (; i + (size_t)(U - 1) * blockDim.x < hi; i += (size_t)U * blockDim.x) {
+  // every pass issues U loads per thread; past the end of the span a thread re-reads the span's last vector (cached)
+  // and drops it, so the tail of a span costs one pass like any other instead of a chain of single loads
+  for (size_t i = lo + threadIdx.x; i < hi; i += (size_t)U * blockDim.x) {
     u32x4 v[U];
 #pragma unroll
-    for (int u = 0; u < U; u++) v[u] = load_stream(src + i + (size_t)u * blockDim.x);
+    for (int u = 0; u < U; u++) {
+      const size_t j = i + (size_t)u * blockDim.x;
+      v[u] = load_stream(src + (j < hi ? j : hi - 1));
+    }
 #pragma unroll
-    for (int u = 0; u < U; u++) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
-  }
-  for (; i < hi; i += blockDim.x) {
-    const u32x4 v = load_stream(src + i);
-    acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    for (int u = 0; u < U; u++) {
+      const size_t j = i + (size_t)u * blockDim.x;
+      if (j < hi) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
   }
   if (acc == never) *sink = acc;
 }
