@@ -54,9 +54,8 @@ def flag_gemv_gemv_triton(x, Wgate, Wup, Wdownt, threshold):
     """Gate in torch (``x @ Wgate``, Wgate (H, I)), then sparse up / down (reference __init__.py:38-43)."""
     act_fn = torch.nn.SiLU()
     x_1 = act_fn(torch.matmul(x, Wgate))
-    flags = torch.abs(x_1) > threshold
-    x = gather_gemv_elemul_flag_3d(x, x_1, Wup, flags)
-    return gather_transposed_gemv_flag_3d(x, Wdownt, flags)
+    # flags = |x_1| > threshold, sparse up, sparse down: one call (the flags are derived where x_1 is read)
+    return gemv_gemv_triton(x, x_1, Wup, Wdownt, threshold)
 
 
 def gemv_gemv_triton(x, x_1, Wup, Wdownt, threshold):
