@@ -703,7 +703,8 @@ def test_norm_and_residual_folded_into_the_mlp(oracle, H, I, B, dtype):
 
 
 @pytest.mark.parametrize("H,I,B,dtype", [(4096, 11008, 1, torch.float16), (4096, 1000, 2, torch.bfloat16), (512, 768, 4, torch.float16),
-                                         (1024, 640, 8, torch.bfloat16), (256, 333, 3, torch.float32), (2048, 512, 12, torch.float16)])
+                                         (1024, 640, 8, torch.bfloat16), (256, 333, 3, torch.float32), (2048, 512, 12, torch.float16),
+                                         (256, 200, 10, torch.float32), (1056, 300, 9, torch.bfloat16)])   # the last two: two passes of <= 8 rows
 def test_next_norm_written_by_the_finishing_launch(oracle, H, I, B, dtype):
     """cats_mlp_norm_residual_norm: `out` carries the bits of cats_mlp_norm_residual (same launches), and `next` is the
     RMS norm of exactly those stored values -- checked against the restated HF norm evaluated on the kernel's own `out`
