@@ -122,7 +122,8 @@ __global__ __launch_bounds__(1024) void union_count_kernel(const uint8_t* __rest
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct WsLayout {
-  size_t counters, mask, z32, zt, partial, atmp, fin, total;
+  size_t counters, mask, ubytes, z32, zt, partial, atmp, fin, total;
+  bool mask_bytes = false;  // not part of the carving: the pass that just ran left the union of the flags in `ubytes`, not `mask`
 };
 
 constexpr int kMaxGroups = 64;  // neuron groups of the sparse down kernel; bounds the partial-sum scratch
@@ -136,6 +137,7 @@ WsLayout ws_layout(int H, int I) {
   l.counters = o; o += kCounterBytes;
   l.partial = o;  o += align_up((size_t)kMaxGroups * B * ((size_t)(H + 511) / 512 * 512) * 4, 256);
   l.mask = o;     o += align_up((size_t)((I + 63) / 64) * 8, 256);
+  l.ubytes = o;   o += align_up((size_t)I + 8, 256);  // the same as a byte per neuron, read eight at a time
   l.z32 = o;      o += align_up((size_t)CATS_MAX_BATCH * I * 4, 256);  // 16 rows: the one-pass gate + up of 9..16 rows fills it whole
   l.zt = o;       o += align_up((size_t)B * I * 4, 256);
   l.atmp = o;     o += align_up((size_t)B * I * 4, 256);
@@ -231,6 +233,14 @@ void fill_rows(RowsArgs& a, const void* x, const void* w, int K, int N, int nb, 
   a.nch = (a.row_vecs + kWave - 1) / kWave;
 }
 
+// Whether do_rows' pass writes the union of the flags as bytes (a.ubytes_out, the matrix-core kernel) rather than as bits
+// (a.mask_out); the down pass that follows has to be told (WsLayout::mask_bytes).
+bool rows_mask_is_bytes(int mode, int dtype, RowsArgs a) {
+  a.mma = g_tuning.gate_variant >= 0;
+  const int bt = batch_template(a.nb);
+  return dtype == CATS_F16 ? rows_takes_mma<F16>(mode, bt, a) : dtype == CATS_BF16 ? rows_takes_mma<BF16>(mode, bt, a) : false;
+}
+
 int do_rows(int mode, int dtype, const RowsArgs& a_in, hipStream_t s) {
   RowsArgs a = a_in;
   a.mma = g_tuning.gate_variant >= 0;  // gate_variant < 0: keep batches of 2..8 on the wave-per-row kernel
@@ -266,7 +276,11 @@ int set_next_norm(ReduceArgs& r, const NextNorm& next, char* ws, const WsLayout&
   return CATS_OK;
 }
 
-// Sparse down over mask words already in the workspace.
+constexpr int kNotTaken = -1;  // internal: the shape or type rules this way out, take the other one
+
+// Sparse down over mask words already in the workspace.  Up to kKernelBatch rows; 16-bit types with an output that goes
+// through partial sums also take up to CATS_MAX_BATCH rows in one pass over W_down^T (matrix-core kernel) -- a call with
+// more than kKernelBatch rows that cannot go that way returns kNotTaken before anything is launched.
 int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_out, int32_t* count_out, int B, int H, int I,
             int dtype, char* ws, const WsLayout& l, hipStream_t s, const void* residual = nullptr, const uint8_t* flags = nullptr,
             const int64_t* idx = nullptr, int M = 0, const void* bias = nullptr, const NextNorm& next = NextNorm()) {
@@ -274,7 +288,8 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   memset(&d, 0, sizeof(d));
   d.wd = (const u32x4*)wdown_t;
   d.z = z;
-  d.mask = (const uint8_t*)(ws + l.mask);
+  d.mask = (const uint8_t*)(ws + (l.mask_bytes ? l.ubytes : l.mask));
+  d.mask_bytes = l.mask_bytes ? 1 : 0;
   d.flags = flags;
   d.idx = idx;
   d.M = M;
@@ -295,42 +310,59 @@ int do_down(const void* z, bool zf32, const void* wdown_t, float* y32, void* y_o
   if (block < 128) block = 128;  // wave 0 builds the index list, the others stage z
   if (block > 1024) block = 1024;
   while (block & (block - 1)) block &= block - 1;  // the fold across waves halves their number per round
-  const int bt = batch_template(B);
+  const int bt = batch_template(B < kKernelBatch ? B : kKernelBatch);
   // about one workgroup per CU over all slabs; more groups if a group's list and z would not fit in LDS
   int ngroup = g_tuning.down_groups > 0 ? g_tuning.down_groups : 256 / d.nslab;
   if (ngroup < 1) ngroup = 1;
   if (ngroup > kMaxGroups) ngroup = kMaxGroups;
+  if (B > kKernelBatch && ngroup > kMaxGroups / 2) ngroup = kMaxGroups / 2;  // the partial sums of 16 rows take twice the room
   const int zcols = idx ? M : I;  // what the groups split: the index list, or the neuron range
   d.chunk = ((zcols + ngroup - 1) / ngroup + 7) / 8 * 8;
-  if ((size_t)d.chunk * (1 + bt) * 4 > 96 * 1024) return CATS_ERR_SHAPE;  // a group's list and z must fit in LDS
+  if ((size_t)d.chunk * (1 + bt) * 4 > 96 * 1024) return B > kKernelBatch ? kNotTaken : CATS_ERR_SHAPE;  // a group's list and z must fit in LDS
   d.ngroup = (zcols + d.chunk - 1) / d.chunk;
 #ifdef CATS_TIMING
   d.tbuf = g_tbuf_down;
 #endif
+  // Three rows and more of a 16-bit type: the matrix-core kernel (gate_variant < 0 or an explicit down_block keep the
+  // wave-per-row-pair kernel, for comparison).
+  bool mma = dtype != CATS_F32 && B >= 3 && d.partial_out && g_tuning.gate_variant >= 0 && g_tuning.down_block == 0;
+  if (mma) mma = dtype == CATS_F16 ? down_mma_supported<F16>(d) : down_mma_supported<BF16>(d);
+  if (B > kKernelBatch && !mma) return kNotTaken;
   hipError_t e;
-  if (dtype == CATS_F16) e = launch_down<F16>(bt, zf32, d, block, s);
+  if (mma) e = dtype == CATS_F16 ? launch_down_mma<F16>(zf32, d, s) : launch_down_mma<BF16>(zf32, d, s);
+  else if (dtype == CATS_F16) e = launch_down<F16>(bt, zf32, d, block, s);
   else if (dtype == CATS_BF16) e = launch_down<BF16>(bt, zf32, d, block, s);
   else e = launch_down<F32>(bt, zf32, d, block, s);
   if (e != hipSuccess) return CATS_ERR_LAUNCH;
   if (!d.partial_out) return CATS_OK;
-  // the groups' partial sums are added by the reduction launch: rounded into y_out (and the residual added), or added to y32
-  ReduceArgs r;
-  memset(&r, 0, sizeof(r));
-  r.partial = d.partial;
-  r.y_out = y_out;
-  r.y32_acc = reduce_into_y32 ? y32 : nullptr;
-  r.residual = residual;
-  r.bias = bias;
-  r.H = H;
-  r.G = d.ngroup;
-  r.BH = B * H;
-  if (int st = set_next_norm(r, next, ws, l)) return st;
-  FusedArgs none;
-  memset(&none, 0, sizeof(none));
-  if (dtype == CATS_F16) e = launch_fused<F16>(1, 0, 2, none, r, s);
-  else if (dtype == CATS_BF16) e = launch_fused<BF16>(1, 0, 2, none, r, s);
-  else e = launch_fused<F32>(1, 0, 2, none, r, s);
-  return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+  // The groups' partial sums are added by the reduction launch: rounded into y_out (and the residual added), or added to
+  // y32.  One launch for all rows, unless it also writes the next norm: its arrival counters cover kKernelBatch rows.
+  const size_t sz = (size_t)elem_size(dtype);
+  const int rows_per = next.out ? kKernelBatch : B;
+  for (int b0 = 0; b0 < B; b0 += rows_per) {
+    const int nb = B - b0 < rows_per ? B - b0 : rows_per;
+    ReduceArgs r;
+    memset(&r, 0, sizeof(r));
+    r.partial = d.partial + (size_t)b0 * H;
+    r.gstride = (size_t)B * H;
+    r.y_out = y_out ? (char*)y_out + (size_t)b0 * H * sz : nullptr;
+    r.y32_acc = reduce_into_y32 ? y32 + (size_t)b0 * H : nullptr;
+    r.residual = residual ? (const char*)residual + (size_t)b0 * H * sz : nullptr;
+    r.bias = bias;
+    r.H = H;
+    r.G = d.ngroup;
+    r.BH = nb * H;
+    NextNorm nx = next;
+    if (nx.out) nx.out = (char*)nx.out + (size_t)b0 * H * sz;
+    if (int st = set_next_norm(r, nx, ws, l)) return st;
+    FusedArgs none;
+    memset(&none, 0, sizeof(none));
+    if (dtype == CATS_F16) e = launch_fused<F16>(1, 0, 2, none, r, s);
+    else if (dtype == CATS_BF16) e = launch_fused<BF16>(1, 0, 2, none, r, s);
+    else e = launch_fused<F32>(1, 0, 2, none, r, s);
+    if (e != hipSuccess) return CATS_ERR_LAUNCH;
+  }
+  return CATS_OK;
 }
 
 int check_ws(const void* ws, size_t ws_bytes, int H, int I, WsLayout& l) {
@@ -649,8 +681,10 @@ static int mlp_pass(const void* x, const void* wgate, const void* wup, const voi
   a.w2 = (const u32x4*)wup;
   a.z32_out = (float*)((char*)ws + l.z32);
   a.mask_out = (uint8_t*)ws + l.mask;
+  a.ubytes_out = (uint8_t*)ws + l.ubytes;
   a.flag_out = flag_out;
   a.t = round_through(dtype, threshold);
+  l.mask_bytes = rows_mask_is_bytes(kGateUp, dtype, a);
   if (stage != 2) {
     st = do_rows(kGateUp, dtype, a, (hipStream_t)stream);
     if (st) return st;
@@ -660,7 +694,6 @@ static int mlp_pass(const void* x, const void* wgate, const void* wup, const voi
   return do_down(a.z32_out, true, wdown_t, acc, y_out, count_out, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
 }
 
-constexpr int kNotTaken = -1;  // mlp_wide: the call has to go the two-pass way
 
 // Whole MLP for 9..16 rows with W_gate and W_up read once: one matrix-core gate + up launch over all rows (two groups of
 // eight), then the sparse down pass per group of eight rows over the union mask of all rows.  Returns kNotTaken when the
@@ -682,6 +715,8 @@ static int mlp_wide(const void* x, const void* norm_weight, float eps, const voi
   a.w2 = (const u32x4*)wup;
   a.z32_out = (float*)((char*)ws + l.z32);
   a.mask_out = (uint8_t*)ws + l.mask;
+  a.ubytes_out = (uint8_t*)ws + l.ubytes;
+  l.mask_bytes = true;  // the matrix-core kernel or nothing
   a.flag_out = flag_out;
   a.t = round_through(dtype, threshold);
   a.norm_w = (const u32x4*)norm_weight;
@@ -694,6 +729,10 @@ static int mlp_wide(const void* x, const void* norm_weight, float eps, const voi
   if (!ok) return kNotTaken;
   const hipError_t e = dtype == CATS_F16 ? launch_rows_mma16<F16>(a, (hipStream_t)stream) : launch_rows_mma16<BF16>(a, (hipStream_t)stream);
   if (e != hipSuccess) return CATS_ERR_LAUNCH;
+  // all rows in one pass over W_down^T where the matrix-core down kernel takes the shape, else a pass per eight rows
+  st = do_down(a.z32_out, true, wdown_t, y_f32, y_out, count_out, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream, residual ? x : nullptr,
+               nullptr, nullptr, 0, nullptr, next);
+  if (st != kNotTaken) return st;
   const size_t sz = esz(dtype);
   for (int b0 = 0; b0 < B; b0 += kKernelBatch) {
     const int nb = B - b0 < kKernelBatch ? B - b0 : kKernelBatch;
@@ -767,9 +806,11 @@ static int mlp_norm_residual_pass(const void* h, const void* norm_weight, float 
   a.w2 = (const u32x4*)wup;
   a.z32_out = (float*)((char*)ws + l.z32);
   a.mask_out = (uint8_t*)ws + l.mask;
+  a.ubytes_out = (uint8_t*)ws + l.ubytes;
   a.t = round_through(dtype, threshold);
   a.norm_w = (const u32x4*)norm_weight;
   a.norm_eps = eps;
+  l.mask_bytes = rows_mask_is_bytes(kGateUp, dtype, a);
   st = do_rows(kGateUp, dtype, a, (hipStream_t)stream);
   if (st) return st;
   return do_down(a.z32_out, true, wdown_t, nullptr, out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream, h, nullptr, nullptr, 0,

@@ -29,7 +29,8 @@ namespace cats {
 struct DownArgs {
   const u32x4* wd;        // (I, H) neuron-major
   const void* z;          // (nb, I) fp32 or dtype
-  const uint8_t* mask;    // ceil(I/8) bytes, bit j = neuron j active for some batch row
+  const uint8_t* mask;    // ceil(I/8) bytes, bit j = neuron j active for some batch row; or, with mask_bytes set, one
+  int mask_bytes;         //   byte per neuron (readable up to the next multiple of eight), nonzero = active
   const uint8_t* flags;   // alternative to mask: (nb, I) flag bytes, OR-ed over the batch on the fly; NULL = use mask
   const int64_t* idx;     // alternative to both: an index list of M weight rows (any order, duplicates add up, entries outside
   int M;                  //   [0, I) contribute nothing); z is then (nb, M), aligned with the list, and the groups split the list
@@ -89,6 +90,105 @@ struct PairAxpy16 {
   }
 };
 
+// First phase of both down kernels.  Wave 0 turns the mask bytes (or flag bytes, or the given index list) of the range
+// [j0, j1) into an ascending list of weight rows in s_list and leaves their number in *s_n; the other waves copy z of the
+// range, rounded to the storage type, to s_z[b * chunk + (j - j0)] and zero rows nb .. zrows - 1.  The two loads are
+// independent, so the phase costs one memory round trip.  The caller synchronises afterwards.
+template <class DT, bool ZF32>
+__device__ __forceinline__ void down_stage_list_and_z(const DownArgs& p, int j0, int j1, int zcols, bool by_list, int zrows, int* s_list,
+                                                      typename DT::st* s_z, int* s_n) {
+  typedef typename DT::st st;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (wave == 0 && by_list) {
+    // the list is given: entry i of the range is weight row idx[j0 + i]
+    for (int i = lane; i < j1 - j0; i += kWave) {
+      const long long j = p.idx[j0 + i];
+      s_list[i] = (j >= 0 && j < (long long)p.I) ? (int)j : 0;  // an entry outside the matrix reads row 0 against z = 0
+    }
+    if (lane == 0) *s_n = max(j1 - j0, 0);
+  } else if (wave == 0) {
+    int base = 0;
+    for (int byte0 = j0 >> 3; byte0 * 8 < j1; byte0 += kWave) {
+      const int byte = byte0 + lane;
+      uint32_t bits = 0;
+      if (byte * 8 < j1) {
+        if (p.flags) {  // uniform: per-row flag bytes instead of packed bits
+          for (int e = 0; e < 8; e++) {
+            const int j = byte * 8 + e;
+            uint32_t on = 0;
+            if (j < p.I)
+              for (int b = 0; b < p.nb; b++) on |= p.flags[(size_t)b * p.I + j] != 0 ? 1u : 0u;
+            bits |= on << e;
+          }
+        } else if (p.mask_bytes) {  // uniform
+          const uint2 m8 = *(const uint2*)(p.mask + (size_t)byte * 8);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            bits |= ((m8.x >> (8 * e)) & 0xffu) ? 1u << e : 0u;
+            bits |= ((m8.y >> (8 * e)) & 0xffu) ? 16u << e : 0u;
+          }
+        } else {
+          bits = p.mask[byte];
+        }
+        const int rem = j1 - byte * 8;
+        if (rem < 8) bits &= (1u << rem) - 1u;
+      }
+      const int pc = __popc(bits);
+      int rank = base + wave_scan_inclusive(pc, lane) - pc;
+      while (bits) {
+        const int bit = __builtin_ctz(bits);
+        bits &= bits - 1;
+        s_list[rank++] = byte * 8 + bit;
+      }
+      base = __shfl(rank, kWave - 1, kWave);  // lane 63 ends at base + (set bits of this pass)
+    }
+    if (lane == 0) *s_n = base;
+  } else {
+    // one flat loop over (b, q) so that the loads of all batch rows are in flight together
+    const int span = j1 - j0;
+    const int total = p.nb * span;
+    for (int i = tid - kWave; i < total; i += blockDim.x - kWave) {
+      const int b = i / span, q = i - b * span;
+      const size_t o = (size_t)b * zcols + j0 + q;
+      st zv = ZF32 ? DT::fromf(((const float*)p.z)[o]) : ((const st*)p.z)[o];
+      if (by_list) {
+        const long long j = p.idx[j0 + q];
+        if (!(j >= 0 && j < (long long)p.I)) zv = DT::fromf(0.f);
+      }
+      s_z[b * p.chunk + q] = zv;
+    }
+    for (int i = p.nb * p.chunk + tid - kWave; i < zrows * p.chunk; i += blockDim.x - kWave) s_z[i] = DT::fromf(0.f);
+  }
+}
+
+// Total popcount of the mask, by one workgroup (not on the hot path).  s_tmp: 16 floats of LDS nobody else is using.
+__device__ __forceinline__ void down_count_mask(const DownArgs& p, float* s_tmp) {
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid >> 6;
+  int k = 0;
+  if (p.mask_bytes) {
+    for (int j = tid; j < p.I; j += blockDim.x) k += p.mask[j] != 0;
+  } else {
+    for (int byte = tid; byte * 8 < p.I; byte += blockDim.x) {
+      uint32_t bits = p.mask[byte];
+      const int rem = p.I - byte * 8;
+      if (rem < 8) bits &= (1u << rem) - 1u;
+      k += __popc(bits);
+    }
+  }
+  k = (int)wave_sum((float)k);  // far below 2^24: exact in fp32
+  if (lane == 0) s_tmp[wave] = (float)k;
+  __syncthreads();
+  if (tid == 0) {
+    float tot = 0.f;
+    for (int w = 0; w < (int)(blockDim.x >> 6); w++) tot += s_tmp[w];
+    *p.count_out = (int)tot;
+  }
+}
+
 template <class DT, int B, bool ZF32, int U>
 __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   typedef typename DT::st st;
@@ -119,59 +219,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   CATS_STAMP(0);
 
   // ---- 1. wave 0: mask bytes of the range -> ascending index list; the other waves: z of the range -> LDS ----
-  if (wave == 0 && by_list) {
-    // the list is given: entry i of the range is weight row idx[j0 + i]
-    for (int i = lane; i < j1 - j0; i += kWave) {
-      const long long j = p.idx[j0 + i];
-      s_list[i] = (j >= 0 && j < (long long)p.I) ? (int)j : 0;  // an entry outside the matrix reads row 0 against z = 0
-    }
-    if (lane == 0) s_n = max(j1 - j0, 0);
-  } else if (wave == 0) {
-    int base = 0;
-    for (int byte0 = j0 >> 3; byte0 * 8 < j1; byte0 += kWave) {
-      const int byte = byte0 + lane;
-      uint32_t bits = 0;
-      if (byte * 8 < j1) {
-        if (p.flags) {  // uniform: per-row flag bytes instead of packed bits
-          for (int e = 0; e < 8; e++) {
-            const int j = byte * 8 + e;
-            uint32_t on = 0;
-            if (j < p.I)
-              for (int b = 0; b < p.nb; b++) on |= p.flags[(size_t)b * p.I + j] != 0 ? 1u : 0u;
-            bits |= on << e;
-          }
-        } else {
-          bits = p.mask[byte];
-        }
-        const int rem = j1 - byte * 8;
-        if (rem < 8) bits &= (1u << rem) - 1u;
-      }
-      const int pc = __popc(bits);
-      int rank = base + wave_scan_inclusive(pc, lane) - pc;
-      while (bits) {
-        const int bit = __builtin_ctz(bits);
-        bits &= bits - 1;
-        s_list[rank++] = byte * 8 + bit;
-      }
-      base = __shfl(rank, kWave - 1, kWave);  // lane 63 ends at base + (set bits of this pass)
-    }
-    if (lane == 0) s_n = base;
-  } else {
-    // one flat loop over (b, q) so that the loads of all batch rows are in flight together
-    const int span = j1 - j0;
-    const int total = p.nb * span;
-    for (int i = tid - kWave; i < total; i += blockDim.x - kWave) {
-      const int b = i / span, q = i - b * span;
-      const size_t o = (size_t)b * zcols + j0 + q;
-      st zv = ZF32 ? DT::fromf(((const float*)p.z)[o]) : ((const st*)p.z)[o];
-      if (by_list) {
-        const long long j = p.idx[j0 + q];
-        if (!(j >= 0 && j < (long long)p.I)) zv = DT::fromf(0.f);
-      }
-      s_z[b * p.chunk + q] = zv;
-    }
-    for (int i = p.nb * p.chunk + tid - kWave; i < B * p.chunk; i += blockDim.x - kWave) s_z[i] = DT::fromf(0.f);
-  }
+  down_stage_list_and_z<DT, ZF32>(p, j0, j1, zcols, by_list, B, s_list, s_z, &s_n);
   __syncthreads();
   const int n = s_n;
   const int nfull = n >> 1;  // whole pairs; pair k is list entries 2k and 2k + 1
@@ -291,21 +339,7 @@ __global__ __launch_bounds__(1024) void down_kernel(DownArgs p) {
   CATS_STAMP(5);
   if (p.count_out && blockIdx.x == 0) {  // not on the hot path: total popcount of the mask
     __syncthreads();  // s_red is reused below; the fold above may still be reading it
-    int k = 0;
-    for (int byte = tid; byte * 8 < p.I; byte += blockDim.x) {
-      uint32_t bits = p.mask[byte];
-      const int rem = p.I - byte * 8;
-      if (rem < 8) bits &= (1u << rem) - 1u;
-      k += __popc(bits);
-    }
-    k = (int)wave_sum((float)k);  // far below 2^24: exact in fp32
-    if (lane == 0) s_red[wave] = (float)k;
-    __syncthreads();
-    if (tid == 0) {
-      float tot = 0.f;
-      for (int w = 0; w < nwaves; w++) tot += s_red[w];
-      *p.count_out = (int)tot;
-    }
+    down_count_mask(p, s_red);
   }
   CATS_STAMP(3);
 }

@@ -96,7 +96,8 @@ struct FusedArgs {
 };
 
 struct ReduceArgs {
-  const float* partial;  // [G][BH]
+  const float* partial;  // [G][BH]; or [G][gstride] with the BH wanted columns at the front of each, when gstride is set
+  size_t gstride;        // 0 = BH
   const int32_t* counts; // [G]
   void* y_out;           // (nb, H) dtype, flattened to BH
   float* y32_acc;        // instead of y_out: (nb, H) fp32 that the sums are added to, unrounded (the fp32-accumulate contract)
@@ -777,13 +778,14 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(ReduceArgs p) {
   const int col = blockIdx.x * kReduceCols + cq * 4;
   const int per = (p.G + kReduceLanes - 1) / kReduceLanes;
   const int g0 = gl * per, g1 = min(p.G, g0 + per);
+  const size_t gstride = p.gstride ? p.gstride : (size_t)p.BH;
   float4 s = {0.f, 0.f, 0.f, 0.f};
   if (col < p.BH) {
     constexpr int U = 8;
     for (int g = g0; g < g1; g += U) {
       float4 t[U];
 #pragma unroll
-      for (int u = 0; u < U; u++) t[u] = *(const float4*)(p.partial + (size_t)min(g + u, g1 - 1) * p.BH + col);
+      for (int u = 0; u < U; u++) t[u] = *(const float4*)(p.partial + (size_t)min(g + u, g1 - 1) * gstride + col);
 #pragma unroll
       for (int u = 0; u < U; u++)
         if (g + u < g1) { s.x += t[u].x; s.y += t[u].y; s.z += t[u].z; s.w += t[u].w; }

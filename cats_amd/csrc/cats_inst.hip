@@ -61,6 +61,7 @@ template <class DT>
 struct MmaLaunch16 {
   static bool supported(const RowsArgs& a, int ng = 1) {
     const int steps = rows_mma_steps(a.K);
+    if (a.mask_out && !a.ubytes_out) return false;  // this kernel writes the union of the flags as bytes only
     return (steps == 4 || steps == 8) && rows_mma_lds_bytes(a.K, ng) <= 160 * 1024;
   }
   // gate + up for 9..16 batch rows in one pass over the weights
@@ -86,12 +87,17 @@ struct MmaLaunch16 {
 template <> struct MmaLaunch<F16> : MmaLaunch16<F16> {};
 template <> struct MmaLaunch<BF16> : MmaLaunch16<BF16> {};
 
+// Whether a call goes to the matrix-core kernel.  Measured on Llama-7B shapes: at 2 batch rows the wave-per-row kernel is
+// still the faster one (28.4 vs 29.4 us).  The plain gate pass goes the same way as gate + up, so a gate call and a fused
+// call produce the same activations bit for bit.
+template <class DT>
+bool takes_mma(int mode, int bt, const RowsArgs& a) {
+  return (mode == kGateUp || mode == kGate) && bt >= 4 && a.mma && MmaLaunch<DT>::supported(a);
+}
+
 template <class DT, int B>
 hipError_t launch_rows_b(int mode, const RowsArgs& a, hipStream_t stream) {
-  // measured on Llama-7B shapes: at 2 batch rows the wave-per-row kernel is still the faster one (28.4 vs 29.4 us)
-  // The plain gate pass goes the same way, so a gate call and a fused call produce the same activations bit for bit.
-  if ((mode == kGateUp || mode == kGate) && B >= 4 && a.mma && MmaLaunch<DT>::supported(a))
-    return MmaLaunch<DT>::run(a, mode == kGateUp, stream);
+  if (takes_mma<DT>(mode, B, a)) return MmaLaunch<DT>::run(a, mode == kGateUp, stream);
   const size_t lds = (size_t)B * ((a.nch + kCB - 1) / kCB * kCB) * kWave * sizeof(u32x4);
   const bool xlds = lds <= 128 * 1024;
   const bool full = xlds && (a.K % (kWave * DT::VEC * kCB) == 0);
@@ -131,6 +137,31 @@ hipError_t launch_down_one(const DownArgs& a, int block, hipStream_t stream) {
   return launch_kernel(kern, dim3(a.nslab * a.ngroup), dim3(block), lds, stream, a);
 }
 
+#ifndef CATS_DOWN_MMA_DEPTH
+#define CATS_DOWN_MMA_DEPTH 2
+#endif
+constexpr int kDownMmaDepth = CATS_DOWN_MMA_DEPTH;  // steps of loads a wave of the matrix-core down kernel keeps in flight
+
+template <class DT>
+struct DownMmaLaunch {
+  static bool supported(const DownArgs&) { return false; }
+  static hipError_t run(bool, const DownArgs&, hipStream_t) { return hipErrorInvalidValue; }
+};
+template <class DT>
+struct DownMmaLaunch16 {
+  static bool supported(const DownArgs& a) {
+    return a.partial_out && a.nb >= 1 && a.nb <= 16 && down_mma_lds_bytes(a.chunk, a.nb, kDownMmaDepth) <= 150 * 1024;
+  }
+  static hipError_t run(bool zf32, const DownArgs& a, hipStream_t stream) {
+    const size_t lds = down_mma_lds_bytes(a.chunk, a.nb, kDownMmaDepth);
+    auto kern = zf32 ? down_mma_kernel<DT, true, kDownMmaDepth> : down_mma_kernel<DT, false, kDownMmaDepth>;
+    if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
+    return launch_kernel(kern, dim3(a.nslab * a.ngroup), dim3(kDownMmaThreads), lds, stream, a);
+  }
+};
+template <> struct DownMmaLaunch<F16> : DownMmaLaunch16<F16> {};
+template <> struct DownMmaLaunch<BF16> : DownMmaLaunch16<BF16> {};
+
 template <class DT, int B, bool FULL, int KV, int DW>
 hipError_t launch_fused_one(int grid, const FusedArgs& a, hipStream_t stream) {
   auto kern = mlp_fused_kernel<DT, B, FULL, KV, DW>;
@@ -168,6 +199,15 @@ hipError_t launch_fused<CATS_DT>(int bt, int grid, int stage, const FusedArgs& a
   }
   return hipSuccess;
 }
+
+template <>
+bool rows_takes_mma<CATS_DT>(int mode, int bt, const RowsArgs& a) { return takes_mma<CATS_DT>(mode, bt, a); }
+
+template <>
+bool down_mma_supported<CATS_DT>(const DownArgs& a) { return DownMmaLaunch<CATS_DT>::supported(a); }
+
+template <>
+hipError_t launch_down_mma<CATS_DT>(bool zf32, const DownArgs& a, hipStream_t stream) { return DownMmaLaunch<CATS_DT>::run(zf32, a, stream); }
 
 template <>
 bool rows_mma16_supported<CATS_DT>(const RowsArgs& a) { return a.mma && MmaLaunch<CATS_DT>::supported(a, 2); }

@@ -3,6 +3,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include "cats_down.h"
+#include "cats_down_mma.h"
 #include "cats_fused.h"
 #include "cats_rows.h"
 
@@ -30,6 +31,10 @@ inline hipError_t launch_kernel(K kern, dim3 grid, dim3 block, size_t lds, hipSt
 // Returns hipSuccess or the launch error.  `mode` is a RowsMode; bt (1, 2, 4 or 8) the compile-time batch.
 template <class DT>
 hipError_t launch_rows(int mode, int bt, const RowsArgs& a, hipStream_t stream);
+// Whether launch_rows sends this call to the matrix-core kernel, which writes the union of the flags to a.ubytes_out
+// (a byte per row) instead of a.mask_out (a bit per row).
+template <class DT>
+bool rows_takes_mma(int mode, int bt, const RowsArgs& a);
 
 // Gate + up for 9..16 batch rows in one pass over the weights (matrix-core kernel with two groups of eight rows):
 // whether the shape and type allow it, and the launch.
@@ -40,6 +45,13 @@ hipError_t launch_rows_mma16(const RowsArgs& a, hipStream_t stream);
 
 template <class DT>
 hipError_t launch_down(int bt, bool zf32, const DownArgs& a, int block, hipStream_t stream);
+
+// Sparse down on the matrix cores: 16-bit types, any number of rows up to 16, partial sums out (a.partial_out set).
+// `supported` also checks that a group's list, z and operands fit in LDS.
+template <class DT>
+bool down_mma_supported(const DownArgs& a);
+template <class DT>
+hipError_t launch_down_mma(bool zf32, const DownArgs& a, hipStream_t stream);
 
 // Single-pass MLP for 1 or 2 batch rows.  stage: 0 = both launches, 1 = streaming kernel only, 2 = reduction only.
 template <class DT>

@@ -28,6 +28,8 @@ struct RowsArgs {
   void* a_out;           // kGate: (nb, N) dtype, optional
   uint8_t* flag_out;     // kGate, kGateUp: (nb, N), optional
   uint8_t* mask_out;     // kGate, kGateUp: ceil(N/8) bytes, bit j = OR over the batch of flag[b, j]; optional
+  uint8_t* ubytes_out;   // the matrix-core kernel's form of mask_out: N bytes, byte j = OR over the batch of flag[b, j].  Its
+                         //   workgroups own row ranges that do not end on multiples of eight, so they cannot write whole mask bytes.
   float* z32_out;        // kGateUp: (nb, N) fp32, written for rows fetched from wup only; kUp: fp32 out, all rows
   void* zt_out;          // kGateUp, kUp, kGemv: (nb, N) dtype, every row written (0 where inactive)
   // index-list mode (kUpIndex): row m of the output is weight row row_idx[m]

@@ -13,8 +13,12 @@
 // two quadrants pair mismatched halves and are dropped.
 //
 // Work split.  One persistent workgroup per CU: x is staged once in LDS in operand order (one linear 16-byte
-// read per lane per step).  A workgroup owns tiles blockIdx, blockIdx + grid, ...; its waves split K.  Tiles
-// move through a software pipeline, one per round:
+// read per lane per step).  A workgroup owns ceil(N / grid) consecutive rows -- the same number of weight bytes for
+// every CU; dealing whole tiles instead leaves 96 of 256 workgroups with 6 tiles against 5 at N = 11008, and the kernel
+// ends 3 us after its median workgroup -- cut into tiles of eight, the last one partial (its missing rows fetch
+// nothing).  The rows of a range do not end on multiples of eight, so the union of the flags goes out as one byte
+// per row (ubytes_out) rather than as bits.  The waves of a workgroup split K.  Tiles move through a software
+// pipeline, one per round:
 //   round r:  MFMA on the gate rows of tile r (loaded two rounds ago) -> per-wave partial sums to LDS;
 //             gate loads of tile r + 2 go out; wave 0 adds the partials in wave order, applies SiLU and the
 //             threshold and publishes the tile's union bits; up loads of tile r go out for the active rows only
@@ -76,9 +80,10 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
   float* part_g = (float*)(xs + (size_t)NG * kXGroup);
   float* part_u = part_g + NG * kPartGroup;
 
-  const int ntiles = (p.N + kMmaTileRows - 1) / kMmaTileRows;
-  const int grid = gridDim.x;
-  const int my_tiles = ntiles > (int)blockIdx.x ? (ntiles - blockIdx.x + grid - 1) / grid : 0;
+  const int rows_per = (p.N + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int r0 = min((int)blockIdx.x * rows_per, p.N);  // this workgroup's rows: [r0, r1)
+  const int r1 = min(r0 + rows_per, p.N);
+  const int my_tiles = (r1 - r0 + kMmaTileRows - 1) / kMmaTileRows;
 
   const int s0 = wave * STEPS;  // this wave's first k step
   // this lane's weight row inside a tile and its 16-byte piece of the 128-byte step
@@ -89,15 +94,13 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
   const bool keep = (lane < 32) ? (ncol < 8) : (ncol >= 8);
   const int slot = (lane >> 5) * 16 + ((lane >> 4) & 1) * 8 + (ncol & 7);
 
-  // Loads of tile number `it` of this workgroup, never predicated: rows past N re-read the last row (their sums
-  // are dropped); lanes with nothing to fetch -- tiles past the end, and with use_any the rows whose union bit is
-  // clear -- read the first bytes of the matrix over and over, which stay in cache and move nothing from HBM.
+  // Loads of tile number `it` of this workgroup, never predicated: lanes with nothing to fetch -- rows past the end of
+  // the range, and with use_any the rows whose union bit is clear -- read the first bytes of the matrix over and over,
+  // which stay in cache and move nothing from HBM (their sums are dropped).
   auto issue = [&](const u32x4* __restrict__ w, int it, u32x4 (&dst)[kMmaSteps], bool use_any) {
-    const bool live = it < my_tiles;  // uniform
-    const int tile = live ? blockIdx.x + it * grid : 0;
-    bool mine = live;
-    if (use_any) mine = live && ((s_any >> jl) & 1u);
-    const int row = min(tile * kMmaTileRows + jl, p.N - 1);
+    const int row = r0 + it * kMmaTileRows + jl;
+    bool mine = row < r1;
+    if (use_any) mine = mine && ((s_any >> jl) & 1u);
     const u32x4* src = mine ? w + (size_t)row * p.row_vecs + piece + (size_t)s0 * 8 : w + piece;
     const int stride = mine ? 8 : 0;
 #pragma unroll
@@ -149,14 +152,13 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
       act[g] = valid[g] = false;
     }
     uint32_t bits8 = 0u;
-    const int tile = blockIdx.x + r * grid;
-    const int row = tile * kMmaTileRows + rj;
+    const int row = r0 + r * kMmaTileRows + rj;
     if (wave == 0 && r < my_tiles) {
       uint64_t bal = 0ull;
 #pragma unroll
       for (int g = 0; g < NG; g++) {
         const int b = g * 8 + rb;  // batch row of this thread in group g
-        valid[g] = row < p.N && b < p.nb;
+        valid[g] = row < r1 && b < p.nb;
         const float gr = DT::rnd(reduce(part_g + g * kPartGroup));
         a[g] = DT::rnd(gr / (1.f + expf(-gr)));
         act[g] = valid[g] && fabsf(a[g]) > p.t;
@@ -166,10 +168,8 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
       }
 #pragma unroll
       for (int j = 0; j < 8; j++) bits8 |= ((bal >> (8 * j)) & 0xffull) ? (1u << j) : 0u;
-      if (lane == 0) {
-        s_any = bits8;
-        if (p.mask_out) p.mask_out[tile] = (uint8_t)bits8;
-      }
+      if (lane == 0) s_any = bits8;
+      if (p.ubytes_out && rb == 0 && row < r1) p.ubytes_out[row] = (uint8_t)((bits8 >> rj) & 1u);
     }
     __syncthreads();
     if (!UP) return;

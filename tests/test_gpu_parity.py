@@ -517,14 +517,14 @@ def test_config4_small_batch_union(oracle, B):
 
 MATRIX_CORE = [
     # H, I, B, dtype -- 3..8 batch rows in 16-bit types with a row length of 2048 or 4096 take the matrix-core
-    # gate / gate+up kernel (tiles of 8 rows dealt round-robin to one workgroup per CU)
-    (4096, 1003, 3, torch.float16),    # I not a multiple of 8: the last tile has 3 live rows
+    # gate / gate+up kernel (one workgroup per CU, each with ceil(I / workgroups) consecutive rows in tiles of 8)
+    (4096, 1003, 3, torch.float16),    # 4 rows per workgroup on 256 CUs: half a tile each, the last workgroup has 3 rows
     (4096, 520, 5, torch.bfloat16),
     (2048, 777, 7, torch.float16),
     (2048, 64, 8, torch.bfloat16),
     (4096, 8, 4, torch.float16),       # a single tile
-    (4096, 2056, 6, torch.float16),    # 257 tiles: one workgroup gets two, the rest one
-    (2048, 6152, 4, torch.bfloat16),   # 769 tiles: four rounds on the first workgroup, three on the others
+    (4096, 2056, 6, torch.float16),    # 9 rows per workgroup: a full tile and one row of the next
+    (2048, 6152, 4, torch.bfloat16),   # 25 rows per workgroup: ranges that start and end inside a mask byte
 ]
 
 
@@ -562,6 +562,55 @@ def test_matrix_core_and_wave_per_row_kernels_agree(oracle):
         assert float(dist.max()) <= A_TOL[torch.float16]["atol"] + A_TOL[torch.float16]["rtol"] * abs(t)
     if int(flips.sum()) == 0:
         close(y_m.cpu(), y_w.cpu(), torch.float16)
+
+
+MATRIX_CORE_DOWN = [
+    # H, I, B, dtype -- 3..8 rows of a 16-bit type through the stand-alone sparse down entry point
+    (4096, 11008, 8, torch.float16),   # the benchmark shape: 32 neuron groups of 344
+    (4096, 1003, 3, torch.float16),    # groups of 32 neurons: two steps of sixteen list entries at most
+    (520, 1000, 5, torch.bfloat16),    # rows of 65 vectors: the second slab holds one
+    (2048, 2049, 7, torch.bfloat16),
+    (64, 96, 4, torch.float16),        # one slab of 8 vectors, lists shorter than one step
+    (4096, 40, 6, torch.float16),
+]
+
+
+@pytest.mark.parametrize("H,I,B,dtype", MATRIX_CORE_DOWN)
+def test_matrix_core_down_kernel(H, I, B, dtype):
+    """The sparse down projection of 3..8 rows on the matrix cores against the spelled-out sum in fp64 and against the
+    wave-per-row-pair kernel (an explicit workgroup size pins that one), for mask densities from empty to full, into a
+    dtype output and into the caller's fp32 accumulator.  Weight rows that no batch row uses hold infinities: a row
+    that is skipped, or that only pads the last step of a list, must not reach the output."""
+    g = torch.Generator().manual_seed(H + I + B)
+    wdt = (torch.randn(I, H, generator=g) * 0.05).to(dtype)
+    z_all = torch.randn(B, I, generator=g).to(dtype)
+    ws = _ws(B, H, I)
+    for density in (0.0, 0.03, 0.5, 1.0):
+        flag = torch.rand(B, I, generator=g) < density
+        if density == 0.03:
+            flag[:, 0] = False  # row 0 is what the padding of a list reads
+        z = torch.where(flag, z_all, torch.zeros_like(z_all))
+        w = wdt.clone()
+        dead = ~flag.any(dim=0)
+        w[dead] = float("inf")
+        want = (z.double() @ torch.where(dead[:, None], torch.zeros_like(wdt), wdt).double()).to(dtype)
+        dz, dw, df = z.cuda(), w.cuda(), flag.to(torch.uint8).cuda()
+        print(f"[case] matrix-core-down H={H} I={I} B={B} {dtype} density={density}", flush=True)
+        y = capi.down_flag(dz, dw, df, ws)
+        acc = torch.full((B, H), 2.0, dtype=torch.float32, device="cuda")
+        capi.down_flag(dz, dw, df, ws, accumulate_into=acc)
+        try:
+            capi.set_tuning(0, 0, 1024, 0)
+            y_pair = capi.down_flag(dz, dw, df, ws)
+        finally:
+            capi.set_tuning(0, 0, 0, 0)
+        y_again = capi.down_flag(dz, dw, df, ws)
+        torch.cuda.synchronize()
+        assert torch.isfinite(y.float()).all()
+        close(y.cpu(), want, dtype)
+        close(y_pair.cpu(), want, dtype)
+        close((acc.cpu() - 2.0).to(dtype), want, dtype)
+        assert torch.equal(y, y_again), "the matrix-core down kernel is not reproducible call to call"
 
 
 SINGLE_PASS = [
