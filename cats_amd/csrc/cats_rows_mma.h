@@ -193,8 +193,8 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
   };
 
   CATS_RSTAMP(0);
-  // ---- prologue.  x is fetched and staged before the first weight load goes out, so that its read does not
-  // queue behind the weight requests of the whole machine. -------------------------------------------------------
+  // ---- prologue.  x is requested before the first weight load goes out, so that its read does not queue behind
+  // the weight requests of the whole machine. ---------------------------------------------------------------------
   u32x4 g0[kMmaSteps], g1[kMmaSteps], u0[kMmaSteps], u1[kMmaSteps];
   {
     // nsteps * 64 operand vectors over kMmaThreads threads = STEPS per thread, all loads in flight together;
@@ -209,6 +209,10 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
         const int n = l & 15, g = l >> 4, b = gb * 8 + (n & 7), kh = n >> 3;
         xv[gb][k] = p.x[(size_t)(b < p.nb ? b : 0) * p.row_vecs + step * 8 + kh * 4 + g];
       }
+    // the first gate tile goes out behind x, before x is waited for: it is a memory round trip ahead when the staging is done
+    __builtin_amdgcn_sched_barrier(0);
+    issue(p.w, 0, g0, false);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int gb = 0; gb < NG; gb++)
 #pragma unroll
@@ -217,12 +221,13 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
         const int b = gb * 8 + (i & 7);
         xs[gb * kXGroup + i] = b < p.nb ? xv[gb][k] : zero4();
       }
-    __builtin_amdgcn_sched_barrier(0);
-    issue(p.w, 0, g0, false);
 #pragma unroll
     for (int c = 0; c < kMmaSteps; c++) u1[c] = zero4();  // defined before the first (unused) up product
   }
-  __syncthreads();
+  // a barrier for LDS only: __syncthreads() would also wait for the gate loads in flight
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
   // The second gate tile goes out after the barrier: a wave blocks at issue once the CU's miss queue is full, so
   // everything issued before the barrier delays the moment the staged x becomes usable.
   issue(p.w, 1, g1, false);
