@@ -57,9 +57,9 @@ typedef enum {
   CATS_ERR_SCRATCH = 8     /* cats_mlp_noalloc: the call does not fit the library's built-in scratch */
 } cats_status_t;
 
-#define CATS_MAX_BATCH 16  /* 1..8 rows are one pass over the weights.  9..16 rows: the whole-MLP entry points read W_gate and W_up
-                            * once (16-bit types, rows of 2048 or 4096 elements) and run the sparse down pass per group of eight
-                            * rows; every other case is two passes of at most eight rows */
+#define CATS_MAX_BATCH 16  /* 1..8 rows are one pass over the weights.  9..16 rows: the whole-MLP entry points read all three
+                            * matrices once (16-bit types, rows of 2048 or 4096 elements); every other case is two passes of
+                            * at most eight rows */
 
 /* Library identification / error text.  No reference counterpart (the reference printf()s and exit()s:
  * flash_gemv/csrc/cuda/fuse_gemv_cmp_cuda.cu:25-33,2397-2400). */
@@ -223,8 +223,9 @@ int cats_mlp_stage(int stage, const void* x, const void* wgate, const void* wup,
 int cats_probe_read(const void* src, size_t bytes, uint32_t* sink, void* stream);
 
 /* Launch-shape knobs for experiments; 0 keeps the built-in choice.  gate_variant N > 0 caps the gate / up kernel at N
- * resident workgroups per CU (N < 0 keeps 3..8 rows off the matrix-core kernel); down_groups / down_block set the neuron
- * groups and the workgroup size of the sparse down kernel; path 1 keeps the whole-MLP entry points on the separate gate+up
+ * resident workgroups per CU (N < 0 keeps 3..16 rows off the matrix-core kernels, gate / up and down); down_groups sets the
+ * neuron groups of the sparse down kernels, down_block the workgroup size of the wave-per-row-pair one -- and keeps 3..16 rows
+ * on that kernel, off the matrix-core one; path 1 keeps the whole-MLP entry points on the separate gate+up
  * and sparse-down kernels for every batch size (by default 1..2 rows take the single-pass kernel).  Every setting computes
  * the same function.  Process-global and not synchronised: set it before other threads call in.  Not in the reference. */
 int cats_set_tuning(int gate_variant, int down_groups, int down_block, int path);
