@@ -627,9 +627,11 @@ static int up_flag_pass(const void* x, const void* wup, const void* a_in, const 
   return do_rows(kUp, dtype, a, (hipStream_t)stream);
 }
 
+// B above kKernelBatch: all rows in one pass over W_down^T where the matrix-core down kernel takes the call, else kNotTaken.
 static int down_flag_pass(const void* z, const void* wdown_t, const uint8_t* flag, float* y_f32, void* y_out, int B, int H, int I,
                    int dtype, void* ws, size_t ws_bytes, void* stream) {
-  int st = check_common(B, H, I, dtype);
+  if (B > kKernelBatch && (B > CATS_MAX_BATCH || dtype == CATS_F32)) return kNotTaken;
+  int st = check_common(B < kKernelBatch ? B : kKernelBatch, H, I, dtype);
   if (st) return st;
   if (!z || !wdown_t || !flag || ((y_f32 == nullptr) == (y_out == nullptr))) return CATS_ERR_NULL;
   if (!aligned16(wdown_t)) return CATS_ERR_ALIGN;
@@ -867,6 +869,8 @@ int cats_up_flag(const void* x, const void* wup, const void* a_in, const uint8_t
 int cats_down_flag(const void* z, const void* wdown_t, const uint8_t* flag, float* y_f32, void* y_out, int B, int H, int I,
                    int dtype, void* ws, size_t ws_bytes, void* stream) {
   const size_t sz = esz(dtype);
+  if (B > kKernelBatch)
+    if (const int st = down_flag_pass(z, wdown_t, flag, y_f32, y_out, B, H, I, dtype, ws, ws_bytes, stream); st != kNotTaken) return st;
   return in_passes(B, [&](size_t b0, int nb) {
     return down_flag_pass(at_cbytes(z, b0 * I * sz), wdown_t, (const uint8_t*)at_cbytes((const void*)flag, b0 * I),
                           (float*)at_bytes((void*)y_f32, b0 * H * 4), at_bytes(y_out, b0 * H * sz), nb, H, I, dtype, ws, ws_bytes, stream);

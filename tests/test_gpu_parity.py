@@ -565,19 +565,22 @@ def test_matrix_core_and_wave_per_row_kernels_agree(oracle):
 
 
 MATRIX_CORE_DOWN = [
-    # H, I, B, dtype -- 3..8 rows of a 16-bit type through the stand-alone sparse down entry point
+    # H, I, B, dtype -- 3..16 rows of a 16-bit type through the stand-alone sparse down entry point
     (4096, 11008, 8, torch.float16),   # the benchmark shape: 32 neuron groups of 344
     (4096, 1003, 3, torch.float16),    # groups of 32 neurons: two steps of sixteen list entries at most
     (520, 1000, 5, torch.bfloat16),    # rows of 65 vectors: the second slab holds one
     (2048, 2049, 7, torch.bfloat16),
     (64, 96, 4, torch.float16),        # one slab of 8 vectors, lists shorter than one step
     (4096, 40, 6, torch.float16),
+    (8192, 3584, 5, torch.float16),    # 16 slabs x 16 groups of 224 neurons
+    (4096, 2048, 16, torch.bfloat16),  # 9..16 rows: one pass over W_down^T for all of them
+    (520, 1000, 11, torch.float16),
 ]
 
 
 @pytest.mark.parametrize("H,I,B,dtype", MATRIX_CORE_DOWN)
 def test_matrix_core_down_kernel(H, I, B, dtype):
-    """The sparse down projection of 3..8 rows on the matrix cores against the spelled-out sum in fp64 and against the
+    """The sparse down projection of 3..16 rows on the matrix cores against the spelled-out sum in fp64 and against the
     wave-per-row-pair kernel (an explicit workgroup size pins that one), for mask densities from empty to full, into a
     dtype output and into the caller's fp32 accumulator.  Weight rows that no batch row uses hold infinities: a row
     that is skipped, or that only pads the last step of a list, must not reach the output."""
@@ -600,7 +603,7 @@ def test_matrix_core_down_kernel(H, I, B, dtype):
         acc = torch.full((B, H), 2.0, dtype=torch.float32, device="cuda")
         capi.down_flag(dz, dw, df, ws, accumulate_into=acc)
         try:
-            capi.set_tuning(0, 0, 1024, 0)
+            capi.set_tuning(0, 0, 1024, 0)  # above eight rows: two passes of that kernel
             y_pair = capi.down_flag(dz, dw, df, ws)
         finally:
             capi.set_tuning(0, 0, 0, 0)
@@ -821,8 +824,8 @@ def test_llama70b_shape(oracle, B):
                                          (2048, 1536, 9, torch.bfloat16), (4096, 11008, 12, torch.float16), (4096, 2048, 16, torch.bfloat16)])
 def test_batches_of_nine_to_sixteen_rows(oracle, H, I, B, dtype):
     """The reference's kernels are instantiated up to 16 rows (fuse_gemv_cmp_cuda.cu:2368-2400).  Here 16-bit rows of 2048
-    or 4096 elements take one matrix-core gate + up pass over all rows (W_gate and W_up read once) and the down pass per
-    group of eight rows over the union mask; every other case is two passes of at most 8 rows.  Either way: the full
+    or 4096 elements take one matrix-core gate + up pass and one matrix-core down pass over all rows (every matrix read
+    once, over the union mask of all rows); every other case is two passes of at most 8 rows.  Either way: the full
     parity case, and rows 8.. of the big batch against the same rows run as a batch of their own (same flags, bit for
     bit; outputs to the parity tolerance -- the union of sixteen rows orders the down sums differently)."""
     m = make_mlp(H, I, B, dtype, seed=B + H, corr=0.3)
