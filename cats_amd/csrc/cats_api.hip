@@ -775,6 +775,8 @@ static int up_down_pass(const void* x, const void* a_in, const void* wup, const 
   a.t = round_through(dtype, threshold);
   a.z32_out = (float*)((char*)ws + l.z32);
   a.mask_out = (uint8_t*)ws + l.mask;
+  a.ubytes_out = (uint8_t*)ws + l.ubytes;
+  l.mask_bytes = rows_mask_is_bytes(kUp, dtype, a);
   st = do_rows(kUp, dtype, a, (hipStream_t)stream);
   if (st) return st;
   return do_down(a.z32_out, true, wdown_t, nullptr, y_out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);

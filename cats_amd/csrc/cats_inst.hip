@@ -54,7 +54,9 @@ hipError_t launch_rows_one(const RowsArgs& a, hipStream_t stream) {
 template <class DT>
 struct MmaLaunch {
   static bool supported(const RowsArgs&, int = 1) { return false; }
+  static bool supported_up(const RowsArgs&) { return false; }
   static hipError_t run(const RowsArgs&, bool, hipStream_t) { return hipErrorInvalidValue; }
+  static hipError_t run_up(const RowsArgs&, hipStream_t) { return hipErrorInvalidValue; }
   static hipError_t run16(const RowsArgs&, hipStream_t) { return hipErrorInvalidValue; }
 };
 template <class DT>
@@ -72,6 +74,26 @@ struct MmaLaunch16 {
     if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
     const int ntiles = (a.N + kMmaTileRows - 1) / kMmaTileRows;
     return launch_kernel(kern, dim3(ntiles < cus ? ntiles : cus), dim3(kMmaThreads), lds, stream, a);
+  }
+  // the up pass alone, gate activations given (kUp without flag bytes, fp32 z for the live rows out)
+  static int up_grid(const RowsArgs& a) {
+    const int cus = current_device_cus();
+    const int ntiles = (a.N + kMmaTileRows - 1) / kMmaTileRows;
+    return ntiles < cus ? ntiles : cus;
+  }
+  static int up_rows_pad(const RowsArgs& a) {
+    const int grid = up_grid(a);
+    return ((a.N + grid - 1) / grid + kMmaTileRows - 1) / kMmaTileRows * kMmaTileRows;
+  }
+  static bool supported_up(const RowsArgs& a) {
+    return supported(a) && a.a_in && !a.flag_in && a.z32_out && !a.zt_out && !a.norm_w && a.nb <= 8 &&
+           rows_mma_up_lds_bytes(a.K, up_rows_pad(a)) <= 160 * 1024;
+  }
+  static hipError_t run_up(const RowsArgs& a, hipStream_t stream) {
+    auto kern = rows_mma_steps(a.K) == 8 ? rows_mma_up_kernel<DT, 8> : rows_mma_up_kernel<DT, 4>;
+    const size_t lds = rows_mma_up_lds_bytes(a.K, up_rows_pad(a));
+    if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
+    return launch_kernel(kern, dim3(up_grid(a)), dim3(kMmaThreads), lds, stream, a);
   }
   static hipError_t run(const RowsArgs& a, bool up, hipStream_t stream) {
     const int cus = current_device_cus();  // one workgroup per CU
@@ -92,12 +114,14 @@ template <> struct MmaLaunch<BF16> : MmaLaunch16<BF16> {};
 // call produce the same activations bit for bit.
 template <class DT>
 bool takes_mma(int mode, int bt, const RowsArgs& a) {
-  return (mode == kGateUp || mode == kGate) && bt >= 4 && a.mma && MmaLaunch<DT>::supported(a);
+  if (bt < 4 || !a.mma) return false;
+  if (mode == kUp) return MmaLaunch<DT>::supported_up(a);
+  return (mode == kGateUp || mode == kGate) && MmaLaunch<DT>::supported(a);
 }
 
 template <class DT, int B>
 hipError_t launch_rows_b(int mode, const RowsArgs& a, hipStream_t stream) {
-  if (takes_mma<DT>(mode, B, a)) return MmaLaunch<DT>::run(a, mode == kGateUp, stream);
+  if (takes_mma<DT>(mode, B, a)) return mode == kUp ? MmaLaunch<DT>::run_up(a, stream) : MmaLaunch<DT>::run(a, mode == kGateUp, stream);
   const size_t lds = (size_t)B * ((a.nch + kCB - 1) / kCB * kCB) * kWave * sizeof(u32x4);
   const bool xlds = lds <= 128 * 1024;
   const bool full = xlds && (a.K % (kWave * DT::VEC * kCB) == 0);

@@ -268,4 +268,135 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
   CATS_RSTAMP(7);
 }
 
+// The up pass alone, for callers that bring the gate activations (kUp without flag_in: flags = |a| > t):
+//   z[b, j] = a[b, j] * (x[b] . wup[j])  for the neurons with a flag in any batch row, union of the flags to ubytes_out.
+// Same tiles, operand layout and work split as rows_mma_kernel.  With a given, every tile's union bits are known before
+// the first weight byte moves: the workgroup stages its range of a in LDS, derives the bits of all its tiles, and then
+// streams W_up with two tiles in flight (a ring of two register sets, the loop unrolled by two) and one barrier per tile
+// (the per-wave partial sums alternate between two buffers: wave 0 adds up tile r while the others multiply tile r + 1).
+// dynamic LDS: x operands | two partial buffers | a of the range, [8][rows_pad] in storage type | one byte of bits per tile
+inline size_t rows_mma_up_lds_bytes(int K, int rows_pad) {
+  return rows_mma_lds_bytes(K, 1) + (size_t)8 * rows_pad * 2 + (size_t)(rows_pad / 8 + 15) / 16 * 16;
+}
+
+template <class DT, int STEPS>
+__global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
+  typedef typename DT::st st;
+  static_assert(sizeof(st) == 2, "16-bit types only");
+  extern __shared__ u32x4 xs[];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int nsteps = kMmaWaves * STEPS;
+  constexpr int kXGroup = nsteps * kWave;
+  constexpr int kPartGroup = kMmaWaves * kMmaPart;
+
+  const int rows_per = (p.N + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int rows_pad = (rows_per + kMmaTileRows - 1) / kMmaTileRows * kMmaTileRows;
+  const int r0 = min((int)blockIdx.x * rows_per, p.N);
+  const int r1 = min(r0 + rows_per, p.N);
+  const int my_tiles = (r1 - r0 + kMmaTileRows - 1) / kMmaTileRows;
+  float* part = (float*)(xs + kXGroup);                     // [2][kPartGroup]
+  st* s_a = (st*)(part + 2 * kPartGroup);                   // [8][rows_pad]
+  uint8_t* s_bits = (uint8_t*)(s_a + 8 * rows_pad);         // [rows_pad / 8]
+
+  const int s0 = wave * STEPS;
+  const int jl = lane & 7;
+  const int piece = ((lane >> 3) & 1) * 4 + (lane >> 4);
+  const int ncol = lane & 15;
+  const bool keep = (lane < 32) ? (ncol < 8) : (ncol >= 8);
+  const int slot = (lane >> 5) * 16 + ((lane >> 4) & 1) * 8 + (ncol & 7);
+  const int rj = lane >> 3, rb = lane & 7;
+
+  CATS_RSTAMP(0);
+  // ---- prologue: x -> LDS in operand order (as rows_mma_kernel), a of the range -> LDS, the bits of every tile ----------
+  {
+    u32x4 xv[STEPS];
+#pragma unroll
+    for (int k = 0; k < STEPS; k++) {
+      const int i = tid + k * kMmaThreads;
+      const int step = i >> 6, l = i & 63;
+      const int n = l & 15, g = l >> 4, b = n & 7, kh = n >> 3;
+      xv[k] = p.x[(size_t)(b < p.nb ? b : 0) * p.row_vecs + step * 8 + kh * 4 + g];
+    }
+    const st* ain = (const st*)p.a_in;
+    for (int e = tid; e < 8 * rows_pad; e += kMmaThreads) {
+      const int b = e / rows_pad, j = e - b * rows_pad;
+      s_a[e] = (b < p.nb && r0 + j < r1) ? ain[(size_t)b * p.N + r0 + j] : DT::fromf(0.f);
+    }
+#pragma unroll
+    for (int k = 0; k < STEPS; k++) {
+      const int i = tid + k * kMmaThreads;
+      xs[i] = (i & 7) < p.nb ? xv[k] : zero4();
+    }
+  }
+  __syncthreads();
+  // one thread per row of the range: any batch row over the threshold?  Eight neighbouring lanes make a tile's byte.
+  for (int j0 = 0; j0 < rows_pad; j0 += kMmaThreads) {
+    const int j = j0 + tid;
+    bool any = false;
+    if (j < rows_pad) {
+#pragma unroll
+      for (int b = 0; b < 8; b++) any = any || (b < p.nb && fabsf(DT::tof(s_a[b * rows_pad + j])) > p.t);
+      any = any && r0 + j < r1;  // the padding of the range holds zeros, which a negative threshold would let through
+      if (p.ubytes_out && r0 + j < r1) p.ubytes_out[r0 + j] = any ? 1 : 0;
+    }
+    const uint64_t bal = __ballot(any);
+    if (j < rows_pad && (lane & 7) == 0) s_bits[j >> 3] = (uint8_t)((bal >> (lane & 56)) & 0xffull);
+  }
+  __syncthreads();
+  CATS_RSTAMP(1);
+
+  auto issue = [&](int it, u32x4 (&dst)[STEPS]) {
+    const int row = r0 + it * kMmaTileRows + jl;
+    const uint32_t bits = it < my_tiles ? s_bits[it] : 0u;
+    const bool mine = row < r1 && ((bits >> jl) & 1u);
+    const u32x4* src = mine ? p.w + (size_t)row * p.row_vecs + piece + (size_t)s0 * 8 : p.w + piece;
+    const int stride = mine ? 8 : 0;
+#pragma unroll
+    for (int c = 0; c < STEPS; c++) dst[c] = load_stream(src + c * stride);
+  };
+  auto multiply = [&](const u32x4 (&src)[STEPS], float* dst_part) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < STEPS; c++) acc = Mma<DT>::run(src[c], xs[(s0 + c) * kWave + lane], acc);
+    if (keep) {
+      float* dst = dst_part + wave * kMmaPart + slot;
+#pragma unroll
+      for (int i = 0; i < 4; i++) dst[i * 32] = acc[i];
+    }
+  };
+  auto body = [&](int r, u32x4 (&ring)[STEPS], float* my_part) {
+    multiply(ring, my_part);
+    issue(r + 2, ring);
+    __syncthreads();
+    if (wave == 0 && r < my_tiles) {
+      // one thread per (row rj of the tile, batch row rb): the eight waves' partials in wave order, then z = a * up
+      const int j = r * kMmaTileRows + rj;
+      const int row = r0 + j;
+      const float* src = my_part + (rj & 3) * 32 + (rj >> 2) * 8 + rb;
+      float u = 0.f;
+#pragma unroll
+      for (int w = 0; w < kMmaWaves; w++) u += src[w * kMmaPart] + src[w * kMmaPart + 16];
+      const float a = DT::tof(s_a[rb * rows_pad + j]);
+      const bool live = (s_bits[r] >> rj) & 1u;
+      if (live && row < r1 && rb < p.nb) {
+        const float z = fabsf(a) > p.t ? DT::rnd(a * DT::rnd(u)) : 0.f;
+        p.z32_out[(size_t)rb * p.N + row] = z;
+      }
+    }
+  };
+
+  u32x4 u0[STEPS], u1[STEPS];
+  issue(0, u0);
+  issue(1, u1);
+  // always in pairs (an odd count ends with a tile of dummy loads): a branch around the second body would leave the
+  // compiler with a path on which its counted waits for the ring degrade to "wait for everything"
+  for (int r = 0; r < my_tiles; r += 2) {
+    body(r, u0, part);
+    body(r + 1, u1, part + kPartGroup);
+  }
+  CATS_RSTAMP(7);
+}
+
 }  // namespace cats

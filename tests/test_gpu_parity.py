@@ -238,7 +238,10 @@ def test_batch_rows_are_independent(oracle):
 
 
 @pytest.mark.parametrize("H,I,B,dtype", [(4096, 1000, 1, torch.float16), (520, 333, 3, torch.bfloat16), (260, 96, 8, torch.float32),
-                                         (4096, 11008, 1, torch.float16), (512, 200, 12, torch.float16)])
+                                         (4096, 11008, 1, torch.float16), (512, 200, 12, torch.float16),
+                                         # 3..8 rows of a 16-bit type with rows of 2048 / 4096 elements: the matrix-core up kernel
+                                         (4096, 1003, 3, torch.float16), (2048, 777, 7, torch.bfloat16), (4096, 11008, 4, torch.float16),
+                                         (2048, 64, 8, torch.float16), (4096, 8, 5, torch.bfloat16), (4096, 520, 12, torch.float16)])
 def test_up_down_given_the_gate_activations(oracle, H, I, B, dtype):
     """cats_up_down (the reference's gemv_gemv_triton): the caller supplies a = act(gate(x)); flags = |a| > t are derived
     on the device and must be the ones torch derives; output against the oracle on those activations and flags."""
@@ -257,6 +260,18 @@ def test_up_down_given_the_gate_activations(oracle, H, I, B, dtype):
     y2 = capi.down_flag(z, d["wdt"], flag.cuda(), ws)
     torch.cuda.synchronize()
     close(y.cpu(), y2.cpu(), dtype)
+    # thresholds that keep everything and nothing, and the wave-per-row kernels on the same call
+    for t2 in (-1.0, 1e9):
+        y3 = capi.up_down(d["x"], a.cuda(), d["wu"], d["wdt"], t2, ws)
+        try:
+            capi.set_tuning(-1, 0, 0, 0)
+            y4 = capi.up_down(d["x"], a.cuda(), d["wu"], d["wdt"], t2, ws)
+        finally:
+            capi.set_tuning(0, 0, 0, 0)
+        torch.cuda.synchronize()
+        ref2 = oracle.c_mlp(m["x"], m["wg"], m["wu"], m["wd"], t2, a_in=a, flag_in=torch.abs(a) > t2)
+        close(y3.cpu(), ref2["y"], dtype)
+        close(y4.cpu(), ref2["y"], dtype)
 
 
 def test_gate_compact_list(oracle):
