@@ -75,7 +75,7 @@ struct MmaLaunch16 {
     const int ntiles = (a.N + kMmaTileRows - 1) / kMmaTileRows;
     return launch_kernel(kern, dim3(ntiles < cus ? ntiles : cus), dim3(kMmaThreads), lds, stream, a);
   }
-  // the up pass alone, gate activations given (kUp without flag bytes, fp32 z for the live rows out)
+  // the up pass alone, gate activations given (kUp)
   static int up_grid(const RowsArgs& a) {
     const int cus = current_device_cus();
     const int ntiles = (a.N + kMmaTileRows - 1) / kMmaTileRows;
@@ -86,7 +86,7 @@ struct MmaLaunch16 {
     return ((a.N + grid - 1) / grid + kMmaTileRows - 1) / kMmaTileRows * kMmaTileRows;
   }
   static bool supported_up(const RowsArgs& a) {
-    return supported(a) && a.a_in && !a.flag_in && a.z32_out && !a.zt_out && !a.norm_w && a.nb <= 8 &&
+    return supported(a) && a.a_in && (a.z32_out || a.zt_out) && !a.norm_w && a.nb <= 8 &&
            rows_mma_up_lds_bytes(a.K, up_rows_pad(a)) <= 160 * 1024;
   }
   static hipError_t run_up(const RowsArgs& a, hipStream_t stream) {

@@ -268,15 +268,18 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
   CATS_RSTAMP(7);
 }
 
-// The up pass alone, for callers that bring the gate activations (kUp without flag_in: flags = |a| > t):
-//   z[b, j] = a[b, j] * (x[b] . wup[j])  for the neurons with a flag in any batch row, union of the flags to ubytes_out.
+// The up pass alone, for callers that bring the gate activations (kUp; flags = |a| > t, or the caller's flag bytes):
+//   z[b, j] = a[b, j] * (x[b] . wup[j])  where flag[b, j], else 0; rows of W_up without a flag in any batch row are not read.
+// Out: the union of the flags to ubytes_out (optional); z as fp32 for the rows that were read (flags derived: the sparse
+// down pass that follows reads no others) or for every row (flags given), and / or in the storage type for every row.
 // Same tiles, operand layout and work split as rows_mma_kernel.  With a given, every tile's union bits are known before
 // the first weight byte moves: the workgroup stages its range of a in LDS, derives the bits of all its tiles, and then
 // streams W_up with two tiles in flight (a ring of two register sets, the loop unrolled by two) and one barrier per tile
 // (the per-wave partial sums alternate between two buffers: wave 0 adds up tile r while the others multiply tile r + 1).
-// dynamic LDS: x operands | two partial buffers | a of the range, [8][rows_pad] in storage type | one byte of bits per tile
+// dynamic LDS: x operands | two partial buffers | a of the range, [8][rows_pad] in storage type | its flags, [8][rows_pad] bytes
+// | one byte of union bits per tile
 inline size_t rows_mma_up_lds_bytes(int K, int rows_pad) {
-  return rows_mma_lds_bytes(K, 1) + (size_t)8 * rows_pad * 2 + (size_t)(rows_pad / 8 + 15) / 16 * 16;
+  return rows_mma_lds_bytes(K, 1) + (size_t)8 * rows_pad * 3 + (size_t)(rows_pad / 8 + 15) / 16 * 16;
 }
 
 template <class DT, int STEPS>
@@ -298,7 +301,8 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
   const int my_tiles = (r1 - r0 + kMmaTileRows - 1) / kMmaTileRows;
   float* part = (float*)(xs + kXGroup);                     // [2][kPartGroup]
   st* s_a = (st*)(part + 2 * kPartGroup);                   // [8][rows_pad]
-  uint8_t* s_bits = (uint8_t*)(s_a + 8 * rows_pad);         // [rows_pad / 8]
+  uint8_t* s_f = (uint8_t*)(s_a + 8 * rows_pad);            // [8][rows_pad]
+  uint8_t* s_bits = s_f + 8 * rows_pad;                     // [rows_pad / 8]
 
   const int s0 = wave * STEPS;
   const int jl = lane & 7;
@@ -322,7 +326,11 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
     const st* ain = (const st*)p.a_in;
     for (int e = tid; e < 8 * rows_pad; e += kMmaThreads) {
       const int b = e / rows_pad, j = e - b * rows_pad;
-      s_a[e] = (b < p.nb && r0 + j < r1) ? ain[(size_t)b * p.N + r0 + j] : DT::fromf(0.f);
+      const bool in = b < p.nb && r0 + j < r1;  // the padding of the range and of the batch is never flagged
+      const size_t o = (size_t)b * p.N + r0 + j;
+      const st av = in ? ain[o] : DT::fromf(0.f);
+      s_a[e] = av;
+      s_f[e] = in && (p.flag_in ? p.flag_in[o] != 0 : fabsf(DT::tof(av)) > p.t) ? 1 : 0;
     }
 #pragma unroll
     for (int k = 0; k < STEPS; k++) {
@@ -331,14 +339,13 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
     }
   }
   __syncthreads();
-  // one thread per row of the range: any batch row over the threshold?  Eight neighbouring lanes make a tile's byte.
+  // one thread per row of the range: any batch row flagged?  Eight neighbouring lanes make a tile's byte.
   for (int j0 = 0; j0 < rows_pad; j0 += kMmaThreads) {
     const int j = j0 + tid;
     bool any = false;
     if (j < rows_pad) {
 #pragma unroll
-      for (int b = 0; b < 8; b++) any = any || (b < p.nb && fabsf(DT::tof(s_a[b * rows_pad + j])) > p.t);
-      any = any && r0 + j < r1;  // the padding of the range holds zeros, which a negative threshold would let through
+      for (int b = 0; b < 8; b++) any = any || s_f[b * rows_pad + j] != 0;
       if (p.ubytes_out && r0 + j < r1) p.ubytes_out[r0 + j] = any ? 1 : 0;
     }
     const uint64_t bal = __ballot(any);
@@ -379,10 +386,12 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
 #pragma unroll
       for (int w = 0; w < kMmaWaves; w++) u += src[w * kMmaPart] + src[w * kMmaPart + 16];
       const float a = DT::tof(s_a[rb * rows_pad + j]);
-      const bool live = (s_bits[r] >> rj) & 1u;
-      if (live && row < r1 && rb < p.nb) {
-        const float z = fabsf(a) > p.t ? DT::rnd(a * DT::rnd(u)) : 0.f;
-        p.z32_out[(size_t)rb * p.N + row] = z;
+      const bool live = (s_bits[r] >> rj) & 1u;       // the row was read
+      if (row < r1 && rb < p.nb) {
+        const float z = s_f[rb * rows_pad + j] ? DT::rnd(a * DT::rnd(u)) : 0.f;  // u of a row that was not read is noise: never used
+        const size_t o = (size_t)rb * p.N + row;
+        if (p.z32_out && (live || p.flag_in)) p.z32_out[o] = z;
+        if (p.zt_out) ((st*)p.zt_out)[o] = DT::fromf(z);
       }
     }
   };

@@ -260,6 +260,17 @@ def test_up_down_given_the_gate_activations(oracle, H, I, B, dtype):
     y2 = capi.down_flag(z, d["wdt"], flag.cuda(), ws)
     torch.cuda.synchronize()
     close(y.cpu(), y2.cpu(), dtype)
+    # the sparse up call alone: against the oracle's z, as fp32 (the same values before the last rounding is undone:
+    # z is rounded to the storage type either way), and in place over a (the reference's fuse_flag_gemv_local contract)
+    close(z.cpu(), ref["z"], dtype)
+    z32 = capi.up_flag(d["x"], d["wu"], a.cuda(), flag.cuda(), out_f32=True)
+    a_inplace = a.cuda().clone()
+    capi.check(capi.lib().cats_up_flag(capi._p(d["x"]), capi._p(d["wu"]), capi._p(a_inplace), capi._p(flag.cuda()), capi._p(a_inplace), 0,
+                                       B, H, I, capi.DTYPE_CODE[dtype], capi._stream(a_inplace)), "cats_up_flag in place")
+    torch.cuda.synchronize()
+    assert torch.equal(z32.to(dtype), z)
+    assert torch.equal(a_inplace, z)
+    assert torch.equal(z.cpu()[~flag], torch.zeros_like(z.cpu()[~flag]))
     # thresholds that keep everything and nothing, and the wave-per-row kernels on the same call
     for t2 in (-1.0, 1e9):
         y3 = capi.up_down(d["x"], a.cuda(), d["wu"], d["wdt"], t2, ws)
