@@ -845,6 +845,40 @@ static int mlp_rowmajor_down_pass(const void* x, const void* wgate, const void* 
   return do_rows(kGemv, dtype, g, (hipStream_t)stream);
 }
 
+// The same for 9..16 rows with every matrix read once: the matrix-core gate + up launch over all rows, then the matrix-core
+// GEMV over all rows.  kNotTaken when the type or the shape rules either kernel out.
+static int mlp_rowmajor_down_wide(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out, int B, int H,
+                                  int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
+  if (B <= kKernelBatch || B > CATS_MAX_BATCH || dtype == CATS_F32) return kNotTaken;
+  int st = check_common(kKernelBatch, H, I, dtype);
+  if (st) return st;
+  if (!x || !wgate || !wup || !wdown || !y_out) return CATS_ERR_NULL;
+  if (!aligned16(x) || !aligned16(wgate) || !aligned16(wup) || !aligned16(wdown)) return CATS_ERR_ALIGN;
+  if (((size_t)I * elem_size(dtype)) % 16 != 0) return CATS_ERR_ALIGN;
+  WsLayout l;
+  st = check_ws(ws, ws_bytes, H, I, l);
+  if (st) return st;
+  RowsArgs a;
+  fill_rows(a, x, wgate, H, I, B, dtype);
+  a.w2 = (const u32x4*)wup;
+  a.zt_out = (char*)ws + l.zt;  // 16 rows of a 16-bit type fill the region of 8 rows of fp32
+  a.t = round_through(dtype, threshold);
+  a.mma = g_tuning.gate_variant >= 0;
+  RowsArgs g;
+  fill_rows(g, (char*)ws + l.zt, wdown, I, H, B, dtype);
+  g.zt_out = y_out;
+  g.mma = a.mma;
+#ifdef CATS_TIMING
+  a.tbuf = g_tbuf_rows;
+#endif
+  const bool ok = dtype == CATS_F16 ? rows_mma16_supported<F16>(a) && rows_takes_mma<F16>(kGemv, kKernelBatch, g)
+                                    : rows_mma16_supported<BF16>(a) && rows_takes_mma<BF16>(kGemv, kKernelBatch, g);
+  if (!ok) return kNotTaken;
+  const hipError_t e = dtype == CATS_F16 ? launch_rows_mma16<F16>(a, (hipStream_t)stream) : launch_rows_mma16<BF16>(a, (hipStream_t)stream);
+  if (e != hipSuccess) return CATS_ERR_LAUNCH;
+  return do_rows(kGemv, dtype, g, (hipStream_t)stream);
+}
+
 // ---- public entry points: up to CATS_MAX_BATCH rows, in passes of kKernelBatch rows over the weights --------------
 // Decode batches of 1..8 rows are one pass.  Larger ones (the reference's kernels go to 16) re-read the weights per
 // pass; at that size the union of the masks is dense anyway and the path has nothing left to skip.
@@ -1067,6 +1101,7 @@ int cats_mlp_norm_residual_norm(const void* h, const void* norm_weight, float ep
 int cats_mlp_rowmajor_down(const void* x, const void* wgate, const void* wup, const void* wdown, void* y_out, int B, int H,
                            int I, int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
   const size_t sz = esz(dtype);
+  if (const int st = mlp_rowmajor_down_wide(x, wgate, wup, wdown, y_out, B, H, I, dtype, threshold, ws, ws_bytes, stream); st != kNotTaken) return st;
   return in_passes(B, [&](size_t b0, int nb) {
     return mlp_rowmajor_down_pass(at_cbytes(x, b0 * H * sz), wgate, wup, wdown, at_bytes(y_out, b0 * H * sz), nb, H, I, dtype, threshold, ws,
                                   ws_bytes, stream);

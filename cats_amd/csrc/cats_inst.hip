@@ -55,8 +55,10 @@ template <class DT>
 struct MmaLaunch {
   static bool supported(const RowsArgs&, int = 1) { return false; }
   static bool supported_up(const RowsArgs&) { return false; }
+  static bool supported_gemv(const RowsArgs&) { return false; }
   static hipError_t run(const RowsArgs&, bool, hipStream_t) { return hipErrorInvalidValue; }
   static hipError_t run_up(const RowsArgs&, hipStream_t) { return hipErrorInvalidValue; }
+  static hipError_t run_gemv(const RowsArgs&, hipStream_t) { return hipErrorInvalidValue; }
   static hipError_t run16(const RowsArgs&, hipStream_t) { return hipErrorInvalidValue; }
 };
 template <class DT>
@@ -95,6 +97,18 @@ struct MmaLaunch16 {
     if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
     return launch_kernel(kern, dim3(up_grid(a)), dim3(kMmaThreads), lds, stream, a);
   }
+  // dense GEMV out = x . w^T (kGemv): any row length, 3..16 batch rows
+  static bool supported_gemv(const RowsArgs& a) {
+    return a.zt_out && !a.norm_w && !a.bias && !a.scale && a.nb <= 16 && a.K % DT::VEC == 0 &&
+           gemv_mma_lds_bytes(a.nb > 8 ? 2 : 1, up_rows_pad(a)) <= 160 * 1024;
+  }
+  static hipError_t run_gemv(const RowsArgs& a, hipStream_t stream) {
+    const int ng = a.nb > 8 ? 2 : 1;
+    auto kern = ng == 2 ? gemv_mma_kernel<DT, 2> : gemv_mma_kernel<DT, 1>;
+    const size_t lds = gemv_mma_lds_bytes(ng, up_rows_pad(a));
+    if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
+    return launch_kernel(kern, dim3(up_grid(a)), dim3(kMmaThreads), lds, stream, a);
+  }
   static hipError_t run(const RowsArgs& a, bool up, hipStream_t stream) {
     const int cus = current_device_cus();  // one workgroup per CU
     const bool s8 = rows_mma_steps(a.K) == 8;
@@ -116,12 +130,14 @@ template <class DT>
 bool takes_mma(int mode, int bt, const RowsArgs& a) {
   if (bt < 4 || !a.mma) return false;
   if (mode == kUp) return MmaLaunch<DT>::supported_up(a);
+  if (mode == kGemv) return MmaLaunch<DT>::supported_gemv(a);
   return (mode == kGateUp || mode == kGate) && MmaLaunch<DT>::supported(a);
 }
 
 template <class DT, int B>
 hipError_t launch_rows_b(int mode, const RowsArgs& a, hipStream_t stream) {
-  if (takes_mma<DT>(mode, B, a)) return mode == kUp ? MmaLaunch<DT>::run_up(a, stream) : MmaLaunch<DT>::run(a, mode == kGateUp, stream);
+  if (takes_mma<DT>(mode, B, a))
+    return mode == kUp ? MmaLaunch<DT>::run_up(a, stream) : mode == kGemv ? MmaLaunch<DT>::run_gemv(a, stream) : MmaLaunch<DT>::run(a, mode == kGateUp, stream);
   const size_t lds = (size_t)B * ((a.nch + kCB - 1) / kCB * kCB) * kWave * sizeof(u32x4);
   const bool xlds = lds <= 128 * 1024;
   const bool full = xlds && (a.K % (kWave * DT::VEC * kCB) == 0);

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include "cats_down.h"
 #include "cats_down_mma.h"
+#include "cats_gemv_mma.h"
 #include "cats_fused.h"
 #include "cats_rows.h"
 

@@ -642,6 +642,37 @@ def test_matrix_core_down_kernel(H, I, B, dtype):
         assert torch.equal(y, y_again), "the matrix-core down kernel is not reproducible call to call"
 
 
+@pytest.mark.parametrize("H,I,B,dtype", [(2048, 520, 4, torch.float16), (4096, 11008, 8, torch.bfloat16), (4096, 1000, 16, torch.float16),
+                                         (2048, 2056, 11, torch.bfloat16)])
+def test_rowmajor_down_on_the_matrix_cores(oracle, H, I, B, dtype):
+    """cats_mlp_rowmajor_down (flag_gemv_gemv_inner: W_down in nn.Linear's (H, I) layout, read whole) at 3..16 rows runs its
+    down projection as a matrix-core GEMV over rows of any length, cut into chunks.  Against the oracle on the kernel's
+    own activations and flags; then with infinities in the first bytes of W_down, which the padding loads of that kernel
+    re-read: only output column 0, whose weights they are, may see them."""
+    m = make_mlp(H, I, B, dtype, seed=H + I + B, corr=0.4)
+    a_abs = oracle.c_gate(m["x"], m["wg"], -1.0)[0].float().abs().flatten()
+    t = float(torch.quantile(a_abs, 0.5))
+    d = dev(m)
+    ws = _ws(B, H, I)
+    y = capi.mlp_rowmajor_down(d["x"], d["wg"], d["wu"], d["wd"], t, ws)
+    a, flag = capi.gate_flag(d["x"], d["wg"], t)
+    torch.cuda.synchronize()
+    ref = oracle.c_mlp(m["x"], m["wg"], m["wu"], m["wd"], t, a_in=a.cpu(), flag_in=flag.cpu())
+    close(y.cpu(), ref["y"], dtype)
+    wd_inf = d["wd"].clone()
+    wd_inf[0, :64] = float("inf")
+    y_inf = capi.mlp_rowmajor_down(d["x"], d["wg"], d["wu"], wd_inf, t, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(y_inf[:, 1:], y[:, 1:])
+    try:  # and the wave-per-row kernels on the same call
+        capi.set_tuning(-1, 0, 0, 0)
+        y_w = capi.mlp_rowmajor_down(d["x"], d["wg"], d["wu"], d["wd"], t, ws)
+    finally:
+        capi.set_tuning(0, 0, 0, 0)
+    torch.cuda.synchronize()
+    close(y_w.cpu(), ref["y"], dtype)
+
+
 SINGLE_PASS = [
     # H, I, B, dtype -- every template the single-pass kernel is instantiated for (row length in whole blocks of 512
     # vectors or not, 1 / 2 / 4 vectors of a row per down wave), ranges that end short, fewer neurons than row waves
