@@ -458,7 +458,7 @@ def other_configs(torch, F, capi, L, steps, warmup, which, batches=(2, 4, 8, 16)
     dev = torch.device("cuda:0")
     res = []
 
-    def run(name, Hh, Ii, B, dtype, code, sparsities, heavy_tail=False, corr=0.0, nsets=6):
+    def run(name, Hh, Ii, B, dtype, code, sparsities, heavy_tail=False, corr=0.0, nsets=6, batch_entry_points=False):
         g = torch.Generator(device="cuda").manual_seed(1)
         sz = 2
         sets = []
@@ -511,10 +511,19 @@ def other_configs(torch, F, capi, L, steps, warmup, which, batches=(2, 4, 8, 16)
             prepared32 = [a[:4] + (None, p(y32)) + a[6:] for a in prepared]
             us32 = timed(lambda i: L.cats_mlp(*prepared32[i % nsets])) if contract != "y_out" else float("nan")
             tb = sz * Hh * Ii + 2 * sz * Hh * k + sz * B * (2 * Hh + Ii) + 4 * k + 4
-            res.append(dict(config=name, batch=B, row_sparsity_target=s, union_sparsity=round(1 - k / Ii, 4), us=round(us, 2),
-                            touched_MB=round(tb / 1e6, 1), GBps=round(tb / us * 1e-3, 1), hbm_frac=round(tb / us * 1e-3 / HBM_PEAK_GBPS, 4),
-                            dense_us=round(us_dense, 2), speedup_vs_dense=round(us_dense / us, 3), us_f32_accumulate=round(us32, 2),
-                            hbm_frac_f32_accumulate=round(tb / us32 * 1e-3 / HBM_PEAK_GBPS, 4)))
+            line = dict(config=name, batch=B, row_sparsity_target=s, union_sparsity=round(1 - k / Ii, 4), us=round(us, 2),
+                        touched_MB=round(tb / 1e6, 1), GBps=round(tb / us * 1e-3, 1), hbm_frac=round(tb / us * 1e-3 / HBM_PEAK_GBPS, 4),
+                        dense_us=round(us_dense, 2), speedup_vs_dense=round(us_dense / us, 3), us_f32_accumulate=round(us32, 2),
+                        hbm_frac_f32_accumulate=round(tb / us32 * 1e-3 / HBM_PEAK_GBPS, 4))
+            if batch_entry_points:
+                # the same batch through the two other whole-MLP contracts of the reference: gate activations given
+                # (gemv_gemv_triton; reads W_up and W_down^T rows only) and W_down in nn.Linear's layout, read whole
+                # (flag_gemv_gemv_inner, which the reference instantiates for 1, 2, 8 and 16 rows)
+                acts = [capi.gate_flag(x, st["wg"], t)[0] for st in sets]
+                line["us_up_down_given_gate"] = round(timed(lambda i: capi.up_down(x, acts[i % nsets], sets[i % nsets]["wu"], sets[i % nsets]["wdt"], t, ws)), 2)
+                line["us_rowmajor_down"] = round(timed(lambda i: capi.mlp_rowmajor_down(x, sets[i % nsets]["wg"], sets[i % nsets]["wu"], sets[i % nsets]["wd"], t, ws)), 2)
+                del acts
+            res.append(line)
         del sets
         torch.cuda.empty_cache()
 
@@ -522,7 +531,7 @@ def other_configs(torch, F, capi, L, steps, warmup, which, batches=(2, 4, 8, 16)
         run("mistral7b_bf16_heavy_tail", 4096, 14336, 1, torch.bfloat16, capi.BF16, [0.5, 0.7], heavy_tail=True)
     if "batch" in which:
         for B in batches:
-            run(f"llama7b_fp16_batch{B}_corr0.5", 4096, 11008, B, torch.float16, capi.F16, [0.5], corr=0.5)
+            run(f"llama7b_fp16_batch{B}_corr0.5", 4096, 11008, B, torch.float16, capi.F16, [0.5], corr=0.5, batch_entry_points=contract == "both")
     if "70b" in which:
         # the larger shape the reference smoke-tests (flash_gemv/test/test_fuse_gemv_cmp.py:662-676): 1.4 GB per weight set
         run("llama70b_fp16", 8192, 28672, 1, torch.float16, capi.F16, [0.5], nsets=2)
