@@ -643,9 +643,12 @@ static int down_flag_pass(const void* z, const void* wdown_t, const uint8_t* fla
   return do_down(z, false, wdown_t, acc, y_out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream, nullptr, flag);
 }
 
+// B above kKernelBatch: all rows in one pass over both matrices where the matrix-core kernel takes the call, else kNotTaken.
 static int gate_up_pass(const void* x, const void* wgate, const void* wup, void* out, uint8_t* flag_out, int B, int H, int I,
                  int dtype, float threshold, void* stream) {
-  int st = check_common(B, H, I, dtype);
+  const bool wide = B > kKernelBatch;
+  if (wide && (B > CATS_MAX_BATCH || dtype == CATS_F32)) return kNotTaken;
+  int st = check_common(wide ? kKernelBatch : B, H, I, dtype);
   if (st) return st;
   if (!x || !wgate || !wup || !out) return CATS_ERR_NULL;
   if (!aligned16(x) || !aligned16(wgate) || !aligned16(wup)) return CATS_ERR_ALIGN;
@@ -655,7 +658,14 @@ static int gate_up_pass(const void* x, const void* wgate, const void* wup, void*
   a.zt_out = out;
   a.flag_out = flag_out;
   a.t = round_through(dtype, threshold);
-  return do_rows(kGateUp, dtype, a, (hipStream_t)stream);
+  if (!wide) return do_rows(kGateUp, dtype, a, (hipStream_t)stream);
+  a.mma = g_tuning.gate_variant >= 0;
+#ifdef CATS_TIMING
+  a.tbuf = g_tbuf_rows;
+#endif
+  if (!(dtype == CATS_F16 ? rows_mma16_supported<F16>(a) : rows_mma16_supported<BF16>(a))) return kNotTaken;
+  const hipError_t e = dtype == CATS_F16 ? launch_rows_mma16<F16>(a, (hipStream_t)stream) : launch_rows_mma16<BF16>(a, (hipStream_t)stream);
+  return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
 }
 
 static int mlp_pass(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, float* y_f32,
@@ -916,6 +926,8 @@ int cats_down_flag(const void* z, const void* wdown_t, const uint8_t* flag, floa
 int cats_gate_up(const void* x, const void* wgate, const void* wup, void* out, uint8_t* flag_out, int B, int H, int I,
                  int dtype, float threshold, void* stream) {
   const size_t sz = esz(dtype);
+  if (B > kKernelBatch)
+    if (const int st = gate_up_pass(x, wgate, wup, out, flag_out, B, H, I, dtype, threshold, stream); st != kNotTaken) return st;
   return in_passes(B, [&](size_t b0, int nb) {
     return gate_up_pass(at_cbytes(x, b0 * H * sz), wgate, wup, at_bytes(out, b0 * I * sz), (uint8_t*)at_bytes((void*)flag_out, b0 * I), nb, H, I,
                         dtype, threshold, stream);

@@ -14,9 +14,9 @@
 //
 // Work split.  One persistent workgroup per CU: x is staged once in LDS in operand order (one linear 16-byte
 // read per lane per step).  A workgroup owns ceil(N / grid) consecutive rows -- the same number of weight bytes for
-// every CU; dealing whole tiles instead leaves 96 of 256 workgroups with 6 tiles against 5 at N = 11008, and the kernel
-// ends 3 us after its median workgroup -- cut into tiles of eight, the last one partial (its missing rows fetch
-// nothing).  The rows of a range do not end on multiples of eight, so the union of the flags goes out as one byte
+// every CU; dealing whole tiles instead leaves 96 of 256 workgroups with 6 tiles against 5 at N = 11008 and spreads their
+// ends over 4-6 us instead of 1.3-2 (the kernel's duration is the same: the memory system is the limit) -- cut into
+// tiles of eight, the last one partial (its missing rows fetch nothing).  The rows of a range do not end on multiples of eight, so the union of the flags goes out as one byte
 // per row (ubytes_out) rather than as bits.  The waves of a workgroup split K.  Tiles move through a software
 // pipeline, one per round:
 //   round r:  MFMA on the gate rows of tile r (loaded two rounds ago) -> per-wave partial sums to LDS;

@@ -468,7 +468,8 @@ def test_mask_boundaries_on_the_device(oracle, dtype):
 
 def test_sparse_up_and_down_ops(oracle):
     """The stand-alone flag-driven up / down entry points against the oracle's restatement of the Triton pair."""
-    for (H, I, B, dtype) in ((512, 1024, 1, torch.float16), (1024, 1000, 3, torch.bfloat16), (256, 512, 2, torch.float32), (4096, 1024, 4, torch.float16)):
+    for (H, I, B, dtype) in ((512, 1024, 1, torch.float16), (1024, 1000, 3, torch.bfloat16), (256, 512, 2, torch.float32), (4096, 1024, 4, torch.float16),
+                             (4096, 1024, 12, torch.bfloat16), (2048, 520, 16, torch.float16)):   # 9..16 rows: gate + up and down in one pass each
         m = make_mlp(H, I, B, dtype, seed=41, corr=0.5)
         d = dev(m)
         t = calibrate(m["wg"], [0.6])[0]
