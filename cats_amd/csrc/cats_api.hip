@@ -613,9 +613,12 @@ int cats_read_count(const int32_t* count_dev, void* stream) {
   return *pinned;
 }
 
+// B above kKernelBatch: all rows in one pass over W_up where the matrix-core kernel takes the call, else kNotTaken.
 static int up_flag_pass(const void* x, const void* wup, const void* a_in, const uint8_t* flag, void* out, int out_is_f32, int B,
                  int H, int I, int dtype, void* stream) {
-  int st = check_common(B, H, I, dtype);
+  const bool wide = B > kKernelBatch;
+  if (wide && (B > CATS_MAX_BATCH || dtype == CATS_F32)) return kNotTaken;
+  int st = check_common(wide ? kKernelBatch : B, H, I, dtype);
   if (st) return st;
   if (!x || !wup || !a_in || !flag || !out) return CATS_ERR_NULL;
   if (!aligned16(x) || !aligned16(wup)) return CATS_ERR_ALIGN;
@@ -624,6 +627,7 @@ static int up_flag_pass(const void* x, const void* wup, const void* a_in, const 
   a.a_in = a_in;
   a.flag_in = flag;
   if (out_is_f32) a.z32_out = (float*)out; else a.zt_out = out;
+  if (wide && !rows_mask_is_bytes(kUp, dtype, a)) return kNotTaken;  // i.e. the matrix-core up kernel does not take it
   return do_rows(kUp, dtype, a, (hipStream_t)stream);
 }
 
@@ -759,9 +763,12 @@ static int mlp_wide(const void* x, const void* norm_weight, float eps, const voi
   return CATS_OK;
 }
 
+// B above kKernelBatch: all rows in one pass over both matrices where the matrix-core kernels take the call, else kNotTaken.
 static int up_down_pass(const void* x, const void* a_in, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,
                         int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
-  int st = check_common(B, H, I, dtype);
+  const bool wide = B > kKernelBatch;
+  if (wide && (B > CATS_MAX_BATCH || dtype == CATS_F32)) return kNotTaken;
+  int st = check_common(wide ? kKernelBatch : B, H, I, dtype);
   if (st) return st;
   if (!x || !a_in || !wup || !wdown_t || !y_out) return CATS_ERR_NULL;
   if (!aligned16(x) || !aligned16(wup) || !aligned16(wdown_t)) return CATS_ERR_ALIGN;
@@ -787,9 +794,20 @@ static int up_down_pass(const void* x, const void* a_in, const void* wup, const 
   a.mask_out = (uint8_t*)ws + l.mask;
   a.ubytes_out = (uint8_t*)ws + l.ubytes;
   l.mask_bytes = rows_mask_is_bytes(kUp, dtype, a);
+  if (wide && !l.mask_bytes) return kNotTaken;  // only the matrix-core up kernel takes more than eight rows
   st = do_rows(kUp, dtype, a, (hipStream_t)stream);
   if (st) return st;
-  return do_down(a.z32_out, true, wdown_t, nullptr, y_out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
+  st = do_down(a.z32_out, true, wdown_t, nullptr, y_out, nullptr, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream);
+  if (st != kNotTaken) return st;
+  // z of all rows is there: the down pass per group of eight rows over the union of all flags
+  const size_t sz = esz(dtype);
+  for (int b0 = 0; b0 < B; b0 += kKernelBatch) {
+    const int nb = B - b0 < kKernelBatch ? B - b0 : kKernelBatch;
+    st = do_down(a.z32_out + (size_t)b0 * I, true, wdown_t, nullptr, at_bytes(y_out, (size_t)b0 * H * sz), nullptr, nb, H, I, dtype, (char*)ws, l,
+                 (hipStream_t)stream);
+    if (st) return st;
+  }
+  return CATS_OK;
 }
 
 static int mlp_norm_residual_pass(const void* h, const void* norm_weight, float eps, const void* wgate, const void* wup,
@@ -906,6 +924,8 @@ int cats_gate_flag(const void* x, const void* wgate, void* a_out, uint8_t* flag_
 int cats_up_flag(const void* x, const void* wup, const void* a_in, const uint8_t* flag, void* out, int out_is_f32, int B,
                  int H, int I, int dtype, void* stream) {
   const size_t sz = esz(dtype);
+  if (B > kKernelBatch)
+    if (const int st = up_flag_pass(x, wup, a_in, flag, out, out_is_f32, B, H, I, dtype, stream); st != kNotTaken) return st;
   return in_passes(B, [&](size_t b0, int nb) {
     return up_flag_pass(at_cbytes(x, b0 * H * sz), wup, at_cbytes(a_in, b0 * I * sz), (const uint8_t*)at_cbytes((const void*)flag, b0 * I),
                         at_bytes(out, b0 * I * (out_is_f32 ? 4 : sz)), out_is_f32, nb, H, I, dtype, stream);
@@ -1060,6 +1080,8 @@ int cats_mlp_noalloc(const void* x, const void* wgate, const void* wup, const vo
 int cats_up_down(const void* x, const void* a, const void* wup, const void* wdown_t, void* y_out, int B, int H, int I,
                  int dtype, float threshold, void* ws, size_t ws_bytes, void* stream) {
   const size_t sz = esz(dtype);
+  if (B > kKernelBatch)
+    if (const int st = up_down_pass(x, a, wup, wdown_t, y_out, B, H, I, dtype, threshold, ws, ws_bytes, stream); st != kNotTaken) return st;
   return in_passes(B, [&](size_t b0, int nb) {
     return up_down_pass(at_cbytes(x, b0 * H * sz), at_cbytes(a, b0 * I * sz), wup, wdown_t, at_bytes(y_out, b0 * H * sz), nb, H, I, dtype,
                         threshold, ws, ws_bytes, stream);

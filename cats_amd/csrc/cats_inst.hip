@@ -88,12 +88,16 @@ struct MmaLaunch16 {
     return ((a.N + grid - 1) / grid + kMmaTileRows - 1) / kMmaTileRows * kMmaTileRows;
   }
   static bool supported_up(const RowsArgs& a) {
-    return supported(a) && a.a_in && (a.z32_out || a.zt_out) && !a.norm_w && a.nb <= 8 &&
-           rows_mma_up_lds_bytes(a.K, up_rows_pad(a)) <= 160 * 1024;
+    const int ng = a.nb > 8 ? 2 : 1;
+    return supported(a, ng) && a.a_in && (a.z32_out || a.zt_out) && !a.norm_w && a.nb <= 16 &&
+           rows_mma_up_lds_bytes(a.K, up_rows_pad(a), ng) <= 160 * 1024;
   }
   static hipError_t run_up(const RowsArgs& a, hipStream_t stream) {
-    auto kern = rows_mma_steps(a.K) == 8 ? rows_mma_up_kernel<DT, 8> : rows_mma_up_kernel<DT, 4>;
-    const size_t lds = rows_mma_up_lds_bytes(a.K, up_rows_pad(a));
+    const int ng = a.nb > 8 ? 2 : 1;
+    const bool s8 = rows_mma_steps(a.K) == 8;
+    auto kern = ng == 2 ? (s8 ? rows_mma_up_kernel<DT, 8, 2> : rows_mma_up_kernel<DT, 4, 2>)
+                        : (s8 ? rows_mma_up_kernel<DT, 8, 1> : rows_mma_up_kernel<DT, 4, 1>);
+    const size_t lds = rows_mma_up_lds_bytes(a.K, up_rows_pad(a), ng);
     if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
     return launch_kernel(kern, dim3(up_grid(a)), dim3(kMmaThreads), lds, stream, a);
   }

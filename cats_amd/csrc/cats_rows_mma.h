@@ -276,13 +276,14 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_kernel(RowsArgs p) {
 // the first weight byte moves: the workgroup stages its range of a in LDS, derives the bits of all its tiles, and then
 // streams W_up with two tiles in flight (a ring of two register sets, the loop unrolled by two) and one barrier per tile
 // (the per-wave partial sums alternate between two buffers: wave 0 adds up tile r while the others multiply tile r + 1).
-// dynamic LDS: x operands | two partial buffers | a of the range, [8][rows_pad] in storage type | its flags, [8][rows_pad] bytes
-// | one byte of union bits per tile
-inline size_t rows_mma_up_lds_bytes(int K, int rows_pad) {
-  return rows_mma_lds_bytes(K, 1) + (size_t)8 * rows_pad * 3 + (size_t)(rows_pad / 8 + 15) / 16 * 16;
+// NG = 2 takes 9..16 batch rows: a second x operand in LDS and a second MFMA on the same weight registers.
+// dynamic LDS, per group of eight batch rows: x operands | two partial buffers | a of the range, [8][rows_pad] in storage
+// type | its flags, [8][rows_pad] bytes; then one byte of union bits per tile
+inline size_t rows_mma_up_lds_bytes(int K, int rows_pad, int ng) {
+  return rows_mma_lds_bytes(K, ng) + (size_t)ng * 8 * rows_pad * 3 + (size_t)(rows_pad / 8 + 15) / 16 * 16;
 }
 
-template <class DT, int STEPS>
+template <class DT, int STEPS, int NG>
 __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
   typedef typename DT::st st;
   static_assert(sizeof(st) == 2, "16-bit types only");
@@ -299,10 +300,11 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
   const int r0 = min((int)blockIdx.x * rows_per, p.N);
   const int r1 = min(r0 + rows_per, p.N);
   const int my_tiles = (r1 - r0 + kMmaTileRows - 1) / kMmaTileRows;
-  float* part = (float*)(xs + kXGroup);                     // [2][kPartGroup]
-  st* s_a = (st*)(part + 2 * kPartGroup);                   // [8][rows_pad]
-  uint8_t* s_f = (uint8_t*)(s_a + 8 * rows_pad);            // [8][rows_pad]
-  uint8_t* s_bits = s_f + 8 * rows_pad;                     // [rows_pad / 8]
+  constexpr int NB = NG * 8;                                // batch rows the kernel is laid out for
+  float* part = (float*)(xs + NG * kXGroup);                // [2][NG][kPartGroup]
+  st* s_a = (st*)(part + 2 * NG * kPartGroup);              // [NB][rows_pad]
+  uint8_t* s_f = (uint8_t*)(s_a + NB * rows_pad);           // [NB][rows_pad]
+  uint8_t* s_bits = s_f + NB * rows_pad;                    // [rows_pad / 8]
 
   const int s0 = wave * STEPS;
   const int jl = lane & 7;
@@ -315,16 +317,18 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
   CATS_RSTAMP(0);
   // ---- prologue: x -> LDS in operand order (as rows_mma_kernel), a of the range -> LDS, the bits of every tile ----------
   {
-    u32x4 xv[STEPS];
+    u32x4 xv[NG][STEPS];
 #pragma unroll
-    for (int k = 0; k < STEPS; k++) {
-      const int i = tid + k * kMmaThreads;
-      const int step = i >> 6, l = i & 63;
-      const int n = l & 15, g = l >> 4, b = n & 7, kh = n >> 3;
-      xv[k] = p.x[(size_t)(b < p.nb ? b : 0) * p.row_vecs + step * 8 + kh * 4 + g];
-    }
+    for (int gb = 0; gb < NG; gb++)
+#pragma unroll
+      for (int k = 0; k < STEPS; k++) {
+        const int i = tid + k * kMmaThreads;
+        const int step = i >> 6, l = i & 63;
+        const int n = l & 15, g = l >> 4, b = gb * 8 + (n & 7), kh = n >> 3;
+        xv[gb][k] = p.x[(size_t)(b < p.nb ? b : 0) * p.row_vecs + step * 8 + kh * 4 + g];
+      }
     const st* ain = (const st*)p.a_in;
-    for (int e = tid; e < 8 * rows_pad; e += kMmaThreads) {
+    for (int e = tid; e < NB * rows_pad; e += kMmaThreads) {
       const int b = e / rows_pad, j = e - b * rows_pad;
       const bool in = b < p.nb && r0 + j < r1;  // the padding of the range and of the batch is never flagged
       const size_t o = (size_t)b * p.N + r0 + j;
@@ -333,10 +337,12 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
       s_f[e] = in && (p.flag_in ? p.flag_in[o] != 0 : fabsf(DT::tof(av)) > p.t) ? 1 : 0;
     }
 #pragma unroll
-    for (int k = 0; k < STEPS; k++) {
-      const int i = tid + k * kMmaThreads;
-      xs[i] = (i & 7) < p.nb ? xv[k] : zero4();
-    }
+    for (int gb = 0; gb < NG; gb++)
+#pragma unroll
+      for (int k = 0; k < STEPS; k++) {
+        const int i = tid + k * kMmaThreads;
+        xs[gb * kXGroup + i] = gb * 8 + (i & 7) < p.nb ? xv[gb][k] : zero4();
+      }
   }
   __syncthreads();
   // one thread per row of the range: any batch row flagged?  Eight neighbouring lanes make a tile's byte.
@@ -345,7 +351,7 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
     bool any = false;
     if (j < rows_pad) {
 #pragma unroll
-      for (int b = 0; b < 8; b++) any = any || s_f[b * rows_pad + j] != 0;
+      for (int b = 0; b < NB; b++) any = any || s_f[b * rows_pad + j] != 0;
       if (p.ubytes_out && r0 + j < r1) p.ubytes_out[r0 + j] = any ? 1 : 0;
     }
     const uint64_t bal = __ballot(any);
@@ -364,13 +370,16 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
     for (int c = 0; c < STEPS; c++) dst[c] = load_stream(src + c * stride);
   };
   auto multiply = [&](const u32x4 (&src)[STEPS], float* dst_part) {
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < STEPS; c++) acc = Mma<DT>::run(src[c], xs[(s0 + c) * kWave + lane], acc);
-    if (keep) {
-      float* dst = dst_part + wave * kMmaPart + slot;
+    for (int gb = 0; gb < NG; gb++) {
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < 4; i++) dst[i * 32] = acc[i];
+      for (int c = 0; c < STEPS; c++) acc = Mma<DT>::run(src[c], xs[gb * kXGroup + (s0 + c) * kWave + lane], acc);
+      if (keep) {
+        float* dst = dst_part + gb * kPartGroup + wave * kMmaPart + slot;
+#pragma unroll
+        for (int i = 0; i < 4; i++) dst[i * 32] = acc[i];
+      }
     }
   };
   auto body = [&](int r, u32x4 (&ring)[STEPS], float* my_part) {
@@ -381,17 +390,21 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
       // one thread per (row rj of the tile, batch row rb): the eight waves' partials in wave order, then z = a * up
       const int j = r * kMmaTileRows + rj;
       const int row = r0 + j;
-      const float* src = my_part + (rj & 3) * 32 + (rj >> 2) * 8 + rb;
-      float u = 0.f;
-#pragma unroll
-      for (int w = 0; w < kMmaWaves; w++) u += src[w * kMmaPart] + src[w * kMmaPart + 16];
-      const float a = DT::tof(s_a[rb * rows_pad + j]);
       const bool live = (s_bits[r] >> rj) & 1u;       // the row was read
-      if (row < r1 && rb < p.nb) {
-        const float z = s_f[rb * rows_pad + j] ? DT::rnd(a * DT::rnd(u)) : 0.f;  // u of a row that was not read is noise: never used
-        const size_t o = (size_t)rb * p.N + row;
-        if (p.z32_out && (live || p.flag_in)) p.z32_out[o] = z;
-        if (p.zt_out) ((st*)p.zt_out)[o] = DT::fromf(z);
+#pragma unroll
+      for (int gb = 0; gb < NG; gb++) {
+        const int b = gb * 8 + rb;
+        const float* src = my_part + gb * kPartGroup + (rj & 3) * 32 + (rj >> 2) * 8 + rb;
+        float u = 0.f;
+#pragma unroll
+        for (int w = 0; w < kMmaWaves; w++) u += src[w * kMmaPart] + src[w * kMmaPart + 16];
+        const float a = DT::tof(s_a[b * rows_pad + j]);
+        if (row < r1 && b < p.nb) {
+          const float z = s_f[b * rows_pad + j] ? DT::rnd(a * DT::rnd(u)) : 0.f;  // u of a row that was not read is noise: never used
+          const size_t o = (size_t)b * p.N + row;
+          if (p.z32_out && (live || p.flag_in)) p.z32_out[o] = z;
+          if (p.zt_out) ((st*)p.zt_out)[o] = DT::fromf(z);
+        }
       }
     }
   };
@@ -403,7 +416,7 @@ __global__ __launch_bounds__(kMmaThreads) void rows_mma_up_kernel(RowsArgs p) {
   // compiler with a path on which its counted waits for the ring degrade to "wait for everything"
   for (int r = 0; r < my_tiles; r += 2) {
     body(r, u0, part);
-    body(r + 1, u1, part + kPartGroup);
+    body(r + 1, u1, part + NG * kPartGroup);
   }
   CATS_RSTAMP(7);
 }

@@ -57,10 +57,10 @@ typedef enum {
   CATS_ERR_SCRATCH = 8     /* cats_mlp_noalloc: the call does not fit the library's built-in scratch */
 } cats_status_t;
 
-#define CATS_MAX_BATCH 16  /* 1..8 rows are one pass over the weights.  9..16 rows: the whole-MLP entry points including
-                            * cats_mlp_rowmajor_down, and cats_gate_up (16-bit types, rows of 2048 or 4096 elements),
-                            * and cats_down_flag (16-bit types) still read every matrix once; every other case is two
-                            * passes of at most eight rows */
+#define CATS_MAX_BATCH 16  /* 1..8 rows are one pass over the weights.  9..16 rows: the whole-MLP entry points (cats_mlp, the
+                            * layer-tail calls, cats_up_down, cats_mlp_rowmajor_down), cats_gate_up and cats_up_flag
+                            * (16-bit types, rows of 2048 or 4096 elements) and cats_down_flag (16-bit types) still read
+                            * every matrix once; every other case is two passes of at most eight rows */
 
 /* Library identification / error text.  No reference counterpart (the reference printf()s and exit()s:
  * flash_gemv/csrc/cuda/fuse_gemv_cmp_cuda.cu:25-33,2397-2400). */
