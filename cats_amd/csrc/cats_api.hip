@@ -538,9 +538,24 @@ int cats_workspace_init(void* ws, size_t ws_bytes, void* stream) {
   return launch_kernel(fill_zero_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (u32x4*)ws, n16) == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
 }
 
+// Launches the matrix-core kernel for 9..16 rows (gate + up when a.w2 is set, else the gate pass); kNotTaken if it does
+// not take the shape.
+static int rows_wide(RowsArgs& a, int dtype, void* stream) {
+  a.mma = g_tuning.gate_variant >= 0;
+#ifdef CATS_TIMING
+  a.tbuf = g_tbuf_rows;
+#endif
+  if (!(dtype == CATS_F16 ? rows_mma16_supported<F16>(a) : rows_mma16_supported<BF16>(a))) return kNotTaken;
+  const hipError_t e = dtype == CATS_F16 ? launch_rows_mma16<F16>(a, (hipStream_t)stream) : launch_rows_mma16<BF16>(a, (hipStream_t)stream);
+  return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+}
+
+// B above kKernelBatch: all rows in one pass over W_gate where the matrix-core kernel takes the call, else kNotTaken.
 static int gate_flag_pass(const void* x, const void* wgate, void* a_out, uint8_t* flag_out, int B, int H, int I, int dtype,
                    float threshold, void* stream) {
-  int st = check_common(B, H, I, dtype);
+  const bool wide = B > kKernelBatch;
+  if (wide && (B > CATS_MAX_BATCH || dtype == CATS_F32)) return kNotTaken;
+  int st = check_common(wide ? kKernelBatch : B, H, I, dtype);
   if (st) return st;
   if (!x || !wgate || (!a_out && !flag_out)) return CATS_ERR_NULL;
   if (!aligned16(x) || !aligned16(wgate)) return CATS_ERR_ALIGN;
@@ -549,7 +564,7 @@ static int gate_flag_pass(const void* x, const void* wgate, void* a_out, uint8_t
   a.a_out = a_out;
   a.flag_out = flag_out;
   a.t = round_through(dtype, threshold);
-  return do_rows(kGate, dtype, a, (hipStream_t)stream);
+  return wide ? rows_wide(a, dtype, stream) : do_rows(kGate, dtype, a, (hipStream_t)stream);
 }
 
 int cats_gate_compact(const void* x, const void* wgate, void* vals_out, int64_t* idx_out, int32_t* count_out, int H, int I,
@@ -662,14 +677,7 @@ static int gate_up_pass(const void* x, const void* wgate, const void* wup, void*
   a.zt_out = out;
   a.flag_out = flag_out;
   a.t = round_through(dtype, threshold);
-  if (!wide) return do_rows(kGateUp, dtype, a, (hipStream_t)stream);
-  a.mma = g_tuning.gate_variant >= 0;
-#ifdef CATS_TIMING
-  a.tbuf = g_tbuf_rows;
-#endif
-  if (!(dtype == CATS_F16 ? rows_mma16_supported<F16>(a) : rows_mma16_supported<BF16>(a))) return kNotTaken;
-  const hipError_t e = dtype == CATS_F16 ? launch_rows_mma16<F16>(a, (hipStream_t)stream) : launch_rows_mma16<BF16>(a, (hipStream_t)stream);
-  return e == hipSuccess ? CATS_OK : CATS_ERR_LAUNCH;
+  return wide ? rows_wide(a, dtype, stream) : do_rows(kGateUp, dtype, a, (hipStream_t)stream);
 }
 
 static int mlp_pass(const void* x, const void* wgate, const void* wup, const void* wdown_t, void* y_out, float* y_f32,
@@ -915,6 +923,8 @@ static int mlp_rowmajor_down_wide(const void* x, const void* wgate, const void* 
 int cats_gate_flag(const void* x, const void* wgate, void* a_out, uint8_t* flag_out, int B, int H, int I, int dtype,
                    float threshold, void* stream) {
   const size_t sz = esz(dtype);
+  if (B > kKernelBatch)
+    if (const int st = gate_flag_pass(x, wgate, a_out, flag_out, B, H, I, dtype, threshold, stream); st != kNotTaken) return st;
   return in_passes(B, [&](size_t b0, int nb) {
     return gate_flag_pass(at_cbytes(x, b0 * H * sz), wgate, at_bytes(a_out, b0 * I * sz), (uint8_t*)at_bytes((void*)flag_out, b0 * I), nb, H, I,
                           dtype, threshold, stream);

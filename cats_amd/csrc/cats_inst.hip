@@ -68,10 +68,12 @@ struct MmaLaunch16 {
     if (a.mask_out && !a.ubytes_out) return false;  // this kernel writes the union of the flags as bytes only
     return (steps == 4 || steps == 8) && rows_mma_lds_bytes(a.K, ng) <= 160 * 1024;
   }
-  // gate + up for 9..16 batch rows in one pass over the weights
+  // gate + up (a.w2 set) or the gate pass alone for 9..16 batch rows in one pass over the weights
   static hipError_t run16(const RowsArgs& a, hipStream_t stream) {
     const int cus = current_device_cus();
-    auto kern = rows_mma_steps(a.K) == 8 ? rows_mma_kernel<DT, 8, true, 2> : rows_mma_kernel<DT, 4, true, 2>;
+    const bool s8 = rows_mma_steps(a.K) == 8;
+    auto kern = a.w2 ? (s8 ? rows_mma_kernel<DT, 8, true, 2> : rows_mma_kernel<DT, 4, true, 2>)
+                     : (s8 ? rows_mma_kernel<DT, 8, false, 2> : rows_mma_kernel<DT, 4, false, 2>);
     const size_t lds = rows_mma_lds_bytes(a.K, 2);
     if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
     const int ntiles = (a.N + kMmaTileRows - 1) / kMmaTileRows;

@@ -37,8 +37,8 @@ hipError_t launch_rows(int mode, int bt, const RowsArgs& a, hipStream_t stream);
 template <class DT>
 bool rows_takes_mma(int mode, int bt, const RowsArgs& a);
 
-// Gate + up for 9..16 batch rows in one pass over the weights (matrix-core kernel with two groups of eight rows):
-// whether the shape and type allow it, and the launch.
+// Gate + up (a.w2 set) or the gate pass alone for 9..16 batch rows in one pass over the weights (matrix-core kernel with
+// two groups of eight rows): whether the shape and type allow it, and the launch.
 template <class DT>
 bool rows_mma16_supported(const RowsArgs& a);
 template <class DT>

@@ -58,7 +58,7 @@ typedef enum {
 } cats_status_t;
 
 #define CATS_MAX_BATCH 16  /* 1..8 rows are one pass over the weights.  9..16 rows: the whole-MLP entry points (cats_mlp, the
-                            * layer-tail calls, cats_up_down, cats_mlp_rowmajor_down), cats_gate_up and cats_up_flag
+                            * layer-tail calls, cats_up_down, cats_mlp_rowmajor_down), cats_gate_flag, cats_gate_up and cats_up_flag
                             * (16-bit types, rows of 2048 or 4096 elements) and cats_down_flag (16-bit types) still read
                             * every matrix once; every other case is two passes of at most eight rows */
 
