@@ -103,18 +103,19 @@ struct MmaLaunch16 {
     if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
     return launch_kernel(kern, dim3(up_grid(a)), dim3(kMmaThreads), lds, stream, a);
   }
-  // dense GEMV out = x . w^T (kGemv): any row length, 3..16 batch rows
+  // dense GEMV out = x . w^T (kGemv): any row length, 3..16 batch rows, up to 64 rows of w per workgroup
   static bool supported_gemv(const RowsArgs& a) {
-    return a.zt_out && !a.norm_w && !a.bias && !a.scale && a.nb <= 16 && a.K % DT::VEC == 0 &&
-           gemv_mma_lds_bytes(a.nb > 8 ? 2 : 1, up_rows_pad(a)) <= 160 * 1024;
+    return a.zt_out && !a.norm_w && !a.bias && !a.scale && a.nb <= 16 && a.K % DT::VEC == 0 && up_rows_pad(a) <= 8 * kMmaTileRows;
   }
-  static hipError_t run_gemv(const RowsArgs& a, hipStream_t stream) {
-    const int ng = a.nb > 8 ? 2 : 1;
-    auto kern = ng == 2 ? gemv_mma_kernel<DT, 2> : gemv_mma_kernel<DT, 1>;
-    const size_t lds = gemv_mma_lds_bytes(ng, up_rows_pad(a));
+  template <int NG>
+  static hipError_t run_gemv_ng(const RowsArgs& a, hipStream_t stream) {
+    const int tiles = up_rows_pad(a) / kMmaTileRows;
+    auto kern = tiles <= 2 ? gemv_mma_kernel<DT, NG, 2> : tiles <= 4 ? gemv_mma_kernel<DT, NG, 4> : gemv_mma_kernel<DT, NG, 8>;
+    const size_t lds = gemv_mma_lds_bytes();
     if (hipError_t e = ensure_dynamic_lds((const void*)kern, lds); e != hipSuccess) return e;
     return launch_kernel(kern, dim3(up_grid(a)), dim3(kMmaThreads), lds, stream, a);
   }
+  static hipError_t run_gemv(const RowsArgs& a, hipStream_t stream) { return a.nb > 8 ? run_gemv_ng<2>(a, stream) : run_gemv_ng<1>(a, stream); }
   static hipError_t run(const RowsArgs& a, bool up, hipStream_t stream) {
     const int cus = current_device_cus();  // one workgroup per CU
     const bool s8 = rows_mma_steps(a.K) == 8;
