@@ -746,14 +746,8 @@ static int mlp_wide(const void* x, const void* norm_weight, float eps, const voi
   a.t = round_through(dtype, threshold);
   a.norm_w = (const u32x4*)norm_weight;
   a.norm_eps = eps;
-  a.mma = g_tuning.gate_variant >= 0;
-#ifdef CATS_TIMING
-  a.tbuf = g_tbuf_rows;
-#endif
-  const bool ok = dtype == CATS_F16 ? rows_mma16_supported<F16>(a) : rows_mma16_supported<BF16>(a);
-  if (!ok) return kNotTaken;
-  const hipError_t e = dtype == CATS_F16 ? launch_rows_mma16<F16>(a, (hipStream_t)stream) : launch_rows_mma16<BF16>(a, (hipStream_t)stream);
-  if (e != hipSuccess) return CATS_ERR_LAUNCH;
+  st = rows_wide(a, dtype, stream);
+  if (st) return st;  // an error, or kNotTaken
   // all rows in one pass over W_down^T where the matrix-core down kernel takes the shape, else a pass per eight rows
   st = do_down(a.z32_out, true, wdown_t, y_f32, y_out, count_out, B, H, I, dtype, (char*)ws, l, (hipStream_t)stream, residual ? x : nullptr,
                nullptr, nullptr, 0, nullptr, next);
@@ -899,19 +893,14 @@ static int mlp_rowmajor_down_wide(const void* x, const void* wgate, const void* 
   a.w2 = (const u32x4*)wup;
   a.zt_out = (char*)ws + l.zt;  // 16 rows of a 16-bit type fill the region of 8 rows of fp32
   a.t = round_through(dtype, threshold);
-  a.mma = g_tuning.gate_variant >= 0;
   RowsArgs g;
   fill_rows(g, (char*)ws + l.zt, wdown, I, H, B, dtype);
   g.zt_out = y_out;
-  g.mma = a.mma;
-#ifdef CATS_TIMING
-  a.tbuf = g_tbuf_rows;
-#endif
-  const bool ok = dtype == CATS_F16 ? rows_mma16_supported<F16>(a) && rows_takes_mma<F16>(kGemv, kKernelBatch, g)
-                                    : rows_mma16_supported<BF16>(a) && rows_takes_mma<BF16>(kGemv, kKernelBatch, g);
-  if (!ok) return kNotTaken;
-  const hipError_t e = dtype == CATS_F16 ? launch_rows_mma16<F16>(a, (hipStream_t)stream) : launch_rows_mma16<BF16>(a, (hipStream_t)stream);
-  if (e != hipSuccess) return CATS_ERR_LAUNCH;
+  g.mma = g_tuning.gate_variant >= 0;
+  // the GEMV first: nothing may have been launched when the call falls back to two passes
+  if (!(dtype == CATS_F16 ? rows_takes_mma<F16>(kGemv, kKernelBatch, g) : rows_takes_mma<BF16>(kGemv, kKernelBatch, g))) return kNotTaken;
+  st = rows_wide(a, dtype, stream);
+  if (st) return st;  // an error, or kNotTaken
   return do_rows(kGemv, dtype, g, (hipStream_t)stream);
 }
 
