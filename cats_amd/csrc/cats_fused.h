@@ -766,7 +766,9 @@ __global__ __launch_bounds__(kFusedThreads) void mlp_fused_kernel(FusedArgs p) {
 
 // y[c] = round(sum over g of partial[g][c]) (+ residual[c]);  c runs over the nb * H flattened outputs.  A workgroup of
 // 256 threads owns kReduceCols columns: 8 threads x float4 across, 32 side by side over contiguous ranges of partials
-// (all loads of a range in flight together), then one thread per column adds the 32 range sums in order.
+// (all loads of a range in flight together), then one thread per column adds the 32 range sums in order.  (128 columns
+// and 8 ranges per workgroup, four times fewer workgroups, is no faster for the 32 partials of the sparse down kernels:
+// +0.8 us per call at 8 rows.)
 template <class DT>
 __global__ __launch_bounds__(256) void reduce_partials_kernel(ReduceArgs p) {
   typedef typename DT::st st;
@@ -780,7 +782,10 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(ReduceArgs p) {
   const int g0 = gl * per, g1 = min(p.G, g0 + per);
   const size_t gstride = p.gstride ? p.gstride : (size_t)p.BH;
   float4 s = {0.f, 0.f, 0.f, 0.f};
-  if (col < p.BH) {
+  if (col < p.BH && per == 1) {
+    // at most one partial per thread (the 32 neuron groups of the sparse down kernels): one load, not a batch of eight
+    if (g0 < g1) s = *(const float4*)(p.partial + (size_t)g0 * gstride + col);
+  } else if (col < p.BH) {
     constexpr int U = 8;
     for (int g = g0; g < g1; g += U) {
       float4 t[U];
