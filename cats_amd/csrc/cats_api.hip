@@ -374,6 +374,7 @@ int check_ws(const void* ws, size_t ws_bytes, int H, int I, WsLayout& l) {
 
 
 constexpr int kFusedMaxGrid = 256;  // partials of 256 workgroups x 2 batch rows fit the workspace's partial-sum region
+constexpr int kFusedPerCU = 16 / kFusedWaves;  // workgroups per CU: 1, or 2 in the 512-thread experiment build (one batch row only)
 
 // Whether the single-pass kernel covers this call, and with what launch shape: one workgroup per CU, each with an
 // equal, contiguous share of the neurons.
@@ -390,6 +391,7 @@ bool fused_eligible(int B, int H, int I, int dtype, FusedArgs& f, int& grid, boo
   if (f.row_vecs > kFusedMaxKV * dw * kWave) return false;
   int maxgrid = current_device_cus();
   if (maxgrid > kFusedMaxGrid) maxgrid = kFusedMaxGrid;
+  if (B == 1) maxgrid *= kFusedPerCU;  // at two rows twice the workgroups would not fit the partial-sum region
   int rpw = (I + maxgrid - 1) / maxgrid;
   if (rpw < 2 * rw) rpw = 2 * rw;  // small matrices: fewer workgroups rather than idle row waves
   grid = (I + rpw - 1) / rpw;

@@ -26,12 +26,18 @@
 
 namespace cats {
 
-constexpr int kFusedWaves = 16;
+// Experiment switch, 16 in the product build: -DCATS_FUSED_WAVES=8 builds the kernel as 512-thread workgroups (half the row
+// waves, half the down waves), launched two per CU with half the neuron share each.
+#ifndef CATS_FUSED_WAVES
+#define CATS_FUSED_WAVES 16
+#endif
+constexpr int kFusedWaves = CATS_FUSED_WAVES;
+static_assert(kFusedWaves == 16 || kFusedWaves == 8, "sixteen waves, or eight for the two-workgroups-per-CU experiment");
 // How the 16 waves split into down waves (each owns 1 / DW of the output columns) and row waves.  A row wave keeps one
 // gate row and one up row in flight and waits out a memory round trip per neuron, so at one batch row twelve of them
 // keep the machine busier than eight (measured: 34.6 against 35.5 us on the Llama layer); at two batch rows the down
 // waves carry twice the arithmetic per fetched row and four of them fall behind (45.6 against 42.6 us).
-constexpr int fused_down_waves(int batch_template) { return batch_template == 1 ? 4 : 8; }
+constexpr int fused_down_waves(int batch_template) { return (batch_template == 1 ? 4 : 8) * kFusedWaves / 16; }
 constexpr int kFusedThreads = kFusedWaves * kWave;
 constexpr int kFusedCB = 8;             // 64-lane chunks (of 16 bytes per lane) per block of row loads
 constexpr int kFusedMaxKV = 4;          // a down wave covers KV * 64 vectors of a row: rows of up to 4 * DW * 64 vectors

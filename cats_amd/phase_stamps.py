@@ -40,6 +40,8 @@ def main() -> None:
     ap.add_argument("--sparsity", type=float, default=0.5)
     ap.add_argument("--calls", type=int, default=24)
     ap.add_argument("--sets", type=int, default=8)
+    ap.add_argument("--workgroups-per-cu", type=int, default=1,
+                    help="2 for a library built with CATS_HIP_DEFINES=-DCATS_FUSED_WAVES=8 (the stamp buffer has a line per workgroup)")
     args = ap.parse_args()
 
     if not TIMING_LIB.exists():
@@ -59,7 +61,7 @@ def main() -> None:
     t = -1.0 if args.sparsity <= 0 else float(torch.kthvalue(act.cpu(), int(args.sparsity * act.numel())).values)
     ws = capi.Workspace(B, H, I)
     y = torch.empty(B, H, dtype=torch.float16, device=dev)
-    grid = torch.cuda.get_device_properties(0).multi_processor_count
+    grid = torch.cuda.get_device_properties(0).multi_processor_count * max(1, args.workgroups_per_cu)
     stamps = torch.zeros(grid * SLOTS, dtype=torch.int64, device=dev)
 
     for i in range(16):                                   # warm-up without stamps
